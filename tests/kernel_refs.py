@@ -139,6 +139,167 @@ class TorchOps:
                 out[t, j] = torch.softmax(s, dim=0) @ v[:, j // group]
         return out.to(q.dtype)
 
+    # ---------------------------------------------------------------- stream norms, shift
+    @staticmethod
+    def _entries(batch):
+        """(entry, first flat token, one past the last, slot, start position) per entry."""
+        qs = batch.q_start.tolist()
+        slots = batch.slot_ids.tolist()
+        pos = batch.positions.tolist()
+        return [(b, qs[b], qs[b + 1], slots[b], pos[qs[b]]) for b in range(batch.num_entries)]
+
+    @staticmethod
+    def _unit(x, eps):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+
+    def bigram_embed(self, table, bigram, norm_w, batch, prev_state, *, scale, buckets,
+                     mul_prev, mul_cur, eps):
+        ids = batch.token_ids.long()
+        rows = torch.empty_like(ids)
+        for b, lo, hi, slot, start in self._entries(batch):
+            for t in range(lo, hi):
+                if t > lo:
+                    prev = int(ids[t - 1])
+                elif start == 0:
+                    prev = None
+                else:
+                    prev = int(prev_state[slot, 0])
+                rows[t] = buckets if prev is None else \
+                    (prev * mul_prev + int(ids[t]) * mul_cur) % buckets
+            prev_state[slot, 0] = int(ids[hi - 1])
+        x = table[ids].float() * scale + bigram[rows].float()
+        return self._unit(x, eps) * norm_w.float()
+
+    def postnorm_add(self, resid, delta, post_w, eps):
+        resid.add_(self._unit(delta.float(), eps) * post_w.float())
+
+    def postnorm_add_norm(self, resid, delta, post_w, post_eps, norm_w, norm_eps, out_dtype):
+        self.postnorm_add(resid, delta, post_w, post_eps)
+        return (self._unit(resid, norm_eps) * norm_w.float()).to(out_dtype)
+
+    def norm_token_shift(self, resid, norm_w, eps, shift_w, batch, state, out_dtype):
+        h = self._unit(resid.float(), eps) * norm_w.float()
+        prev = torch.zeros_like(h)
+        for b, lo, hi, slot, start in self._entries(batch):
+            prev[lo + 1:hi] = h[lo:hi - 1]
+            if start > 0:
+                prev[lo] = state[slot]
+            state[slot] = h[hi - 1]
+        return (h + (prev - h) * shift_w.float()).to(out_dtype)
+
+    def polynorm(self, z, coef, eps, out_dtype):
+        z = z.float()
+        a, b, c, e = [float(v) for v in coef.tolist()]
+        z2 = z * z
+        return (a * self._unit(z, eps) + b * self._unit(z2, eps) + c * self._unit(z2 * z, eps)
+                + e).to(out_dtype)
+
+    # ---------------------------------------------------------------- state-space mixer
+    def conv_silu(self, proj, col, channels, weight, bias, batch, state):
+        taps = weight.shape[1]
+        u = proj[:, col:col + channels].float()
+        out = torch.empty_like(u)
+        for b, lo, hi, slot, start in self._entries(batch):
+            hist = state[slot] if start > 0 else torch.zeros_like(state[slot])
+            full = torch.cat([hist, u[lo:hi]], dim=0)           # [taps-1 + n, C]
+            n = hi - lo
+            acc = bias.float().expand(n, channels).clone()
+            for k in range(taps):
+                acc = acc + full[k:k + n] * weight[:, k].float()
+            out[lo:hi] = acc * torch.sigmoid(acc)
+            if taps > 1:
+                state[slot] = full[full.shape[0] - (taps - 1):]
+        return out
+
+    def ssm_scan(self, xbc, proj, dt_col, dt_bias, a_log, d_skip, batch, state, *, heads, vdim,
+                 state_rows, groups):
+        N = state_rows
+        inner, G = heads * vdim, groups
+        T = xbc.shape[0]
+        x = xbc[:, :inner].view(T, heads, vdim)
+        Bm = xbc[:, inner:inner + G * N].view(T, G, N)
+        Cm = xbc[:, inner + G * N:inner + 2 * G * N].view(T, G, N)
+        dt = torch.nn.functional.softplus(proj[:, dt_col:dt_col + heads].float() + dt_bias.float(),
+                                          threshold=30.0)
+        decay = torch.exp(-torch.exp(a_log.float()) * dt)       # [T, heads]
+        g_of_h = torch.arange(heads, device=xbc.device) // (heads // G)
+        y = torch.empty(T, heads, vdim, dtype=torch.float32, device=xbc.device)
+        for b, lo, hi, slot, start in self._entries(batch):
+            S = state[slot].clone() if start > 0 else torch.zeros_like(state[slot])
+            for t in range(lo, hi):
+                Bh, Ch = Bm[t, g_of_h], Cm[t, g_of_h]           # [heads, N]
+                S = decay[t, :, None, None] * S + \
+                    dt[t, :, None, None] * Bh[:, :, None] * x[t][:, None, :]
+                y[t] = (S * Ch[:, :, None]).sum(1) + d_skip.float()[:, None] * x[t]
+            state[slot] = S
+        return y.view(T, inner)
+
+    def gated_group_norm(self, y, proj, norm_w, groups, eps, out_dtype):
+        T, inner = y.shape
+        z = proj[:, :inner].float()
+        g = y.float() * (z * torch.sigmoid(z))
+        g = self._unit(g.view(T, groups, inner // groups), eps).reshape(T, inner)
+        return (g * norm_w.float()).to(out_dtype)
+
+    # ---------------------------------------------------------------- latent attention
+    @staticmethod
+    def _rotate_pairs(v, positions, freqs, dims):
+        ang = positions.float()[:, None] * freqs.float()[None, :]
+        shape = [v.shape[0]] + [1] * (v.dim() - 2) + [dims // 2]
+        cos, sin = torch.cos(ang).view(shape), torch.sin(ang).view(shape)
+        out = v.clone()
+        a, b = v[..., 0:dims:2], v[..., 1:dims:2]
+        out[..., 0:dims:2] = a * cos - b * sin
+        out[..., 1:dims:2] = b * cos + a * sin
+        return out
+
+    def rotate_interleaved_inplace(self, x, positions, freqs, dims):
+        x.copy_(self._rotate_pairs(x.float(), positions, freqs, dims).to(x.dtype))
+
+    def latent_prepare(self, proj, batch, table, cache, *, q_rank, kv_rank, rot_dim, q_norm,
+                       kv_norm, eps, freqs, rot_dims, out_dtype):
+        proj = proj.float()
+        cq = self._unit(proj[:, :q_rank], eps) * q_norm.float()
+        c = self._unit(proj[:, q_rank:q_rank + kv_rank], eps) * kv_norm.float()
+        kr = self._rotate_pairs(proj[:, q_rank + kv_rank:], batch.positions, freqs, rot_dims)
+        P = cache.page_size
+        pos = batch.positions.long()
+        page = table[batch.entry_of_token.long(), pos // P].long()
+        if (page < 0).any():
+            raise RuntimeError("store to a position whose page was given back")
+        cache.k_pages[page, pos % P] = torch.cat([c, kr], dim=-1).to(cache.k_pages.dtype)
+        return cq.to(out_dtype)
+
+    def latent_query(self, q, w_uk, batch, *, heads, dim, rot_dim, kv_rank, freqs, rot_dims):
+        T = q.shape[0]
+        q = q.float().view(T, heads, dim + rot_dim)
+        uk = w_uk.float().view(heads, dim, kv_rank)
+        ql = torch.einsum("thd,hdr->thr", q[..., :dim], uk)
+        qr = self._rotate_pairs(q[..., dim:], batch.positions, freqs, rot_dims)
+        return torch.cat([ql, qr], dim=-1).contiguous()
+
+    def latent_attention(self, qa, batch, table, cache, *, heads, kv_rank, rot_dim, scale,
+                         window):
+        T = qa.shape[0]
+        P = cache.page_size
+        out = torch.empty(T, heads, kv_rank, dtype=torch.float32, device=qa.device)
+        for t in range(T):
+            b, p = int(batch.entry_of_token[t]), int(batch.positions[t])
+            lo = 0 if window is None else max(0, p - window + 1)
+            keys = torch.arange(lo, p + 1, device=qa.device)
+            pages = table[b, keys // P].long()
+            if (pages < 0).any():
+                raise RuntimeError("attention reads a position whose page was given back")
+            kv = cache.k_pages[pages, keys % P].float()          # [n, kv_rank + rot_dim]
+            s = (kv @ qa[t].float().T) * scale                   # [n, heads]
+            out[t] = torch.softmax(s, dim=0).T @ kv[:, :kv_rank]
+        return out
+
+    def head_linear(self, x, weight, heads, out_dtype):
+        T = x.shape[0]
+        w = weight.float().view(heads, -1, x.shape[-1])          # [heads, out, in]
+        return torch.einsum("thr,hor->tho", x.float(), w).reshape(T, -1).to(out_dtype)
+
     # ---------------------------------------------------------------- sampling
     def argmax(self, logits):
         return logits.float().argmax(dim=-1).to(torch.int32)

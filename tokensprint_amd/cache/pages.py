@@ -140,6 +140,9 @@ class GroupLayout:
     head_dim: int
     window: int | None
     runs: tuple[int, ...]          # run indices whose caches live in this group
+    #: "kv": keys and values per head; "latent": one vector of `head_dim` elements per
+    #: token that every head reads (`num_kv_heads` is 1)
+    kind: str = "kv"
 
 
 @dataclass

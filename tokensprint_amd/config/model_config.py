@@ -34,10 +34,16 @@ def read_config_json(model_dir) -> dict[str, Any]:
 
 
 def architecture_of(raw: dict[str, Any]) -> str:
+    """The architecture a config.json names: the first entry of its 'architectures' list,
+    or its 'architecture' string."""
     archs = raw.get("architectures")
-    if not archs or not isinstance(archs, list):
-        raise ConfigError("config.json has no 'architectures' list; cannot choose a model")
-    return archs[0]
+    if archs and isinstance(archs, list):
+        return archs[0]
+    single = raw.get("architecture")
+    if isinstance(single, str) and single:
+        return single
+    raise ConfigError("config.json has neither an 'architectures' list nor an 'architecture' "
+                      "name; cannot choose a model")
 
 
 @dataclass(frozen=True)

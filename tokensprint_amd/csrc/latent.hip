@@ -1,0 +1,317 @@
+// Attention over a shared low-rank latent kept in pages: every cached token is one row
+// [c (kv_rank) | k_r (rot_dim)] that all heads read, as key (all of it) and as value (c).
+// Queries arrive already carried into that space, q' = [U_k^T q_n | rot(q_r)], and the
+// result leaves as sum_t p_t c_t per head, for the value up-projection behind it.
+//
+// Kernels: the preparation of a step's rows (norms of the two latents, rotation of the
+// shared key part, the write into the pages), the carrying of queries into the latent's
+// space, attention, and the per-head product that carries results back out.
+// Scores, softmax, rotation angles, norms: float32.  The rotation pairs dimension 2i with
+// 2i+1 and turns them by position * freq[i]; cosine and sine are computed here, at the
+// position, so there is no table and no longest position.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(4))) float f32x4_l;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_l;
+__device__ __forceinline__ f32x4_l load4_l(const float* p) { return *(const f32x4_l*)p; }
+__device__ __forceinline__ f32x4_l load4_l(const bf16_t* p) {
+  const bf16x4_l v = *(const bf16x4_l*)p;
+  return f32x4_l{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+}
+
+__device__ __forceinline__ void rotate_pair(float u, float v, int pos, float freq, float* ou,
+                                            float* ov) {
+  float sn, cs;
+  sincosf((float)pos * freq, &sn, &cs);
+  *ou = u * cs - v * sn;
+  *ov = v * cs + u * sn;
+}
+
+// ---------------------------------------------------------------- preparation
+// proj row: [q latent (q_rank) | kv latent (kv_rank) | shared key part (rot_dim)], float32.
+// cq = q latent / rms * q_norm -> out (the up-projection's input);
+// c = kv latent / rms * kv_norm and the rotated key part -> the token's row in the pages.
+template <typename TO, typename TC>
+__global__ __launch_bounds__(256) void latent_prepare_kernel(
+    const float* __restrict__ proj, const float* __restrict__ q_norm,
+    const float* __restrict__ kv_norm, const float* __restrict__ freqs, TO* __restrict__ cq,
+    TC* __restrict__ pages, const int* __restrict__ positions,
+    const int* __restrict__ entry_of_token, const int* __restrict__ table, int table_width,
+    int page_size, int q_rank, int kv_rank, int rot_dim, int rot_dims, float eps) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  const int ld = q_rank + kv_rank + rot_dim, dl = kv_rank + rot_dim;
+  const float* row = proj + (int64_t)t * ld;
+  float sq = 0.f, sc = 0.f;
+  for (int i = threadIdx.x; i < q_rank; i += blockDim.x) sq += row[i] * row[i];
+  for (int i = threadIdx.x; i < kv_rank; i += blockDim.x) sc += row[q_rank + i] * row[q_rank + i];
+  const float rq = 1.0f / sqrtf(block_sum(sq, scratch) / (float)q_rank + eps);
+  const float rc = 1.0f / sqrtf(block_sum(sc, scratch) / (float)kv_rank + eps);
+  TO* o = cq + (int64_t)t * q_rank;
+  for (int i = threadIdx.x; i < q_rank; i += blockDim.x) o[i] = from_f32<TO>(row[i] * rq * q_norm[i]);
+  const int pos = positions[t];
+  const int page = table[(int64_t)entry_of_token[t] * table_width + pos / page_size];
+  if (page < 0) return;     // an idle lane of a fixed-size batch: nothing to keep
+  TC* dst = pages + ((int64_t)page * page_size + pos % page_size) * dl;
+  for (int i = threadIdx.x; i < kv_rank; i += blockDim.x)
+    dst[i] = from_f32<TC>(row[q_rank + i] * rc * kv_norm[i]);
+  const float* kr = row + q_rank + kv_rank;
+  for (int i = threadIdx.x; i < rot_dim / 2 + rot_dim % 2; i += blockDim.x) {
+    if (2 * i + 1 < rot_dims) {
+      float u, v;
+      rotate_pair(kr[2 * i], kr[2 * i + 1], pos, freqs[i], &u, &v);
+      dst[kv_rank + 2 * i] = from_f32<TC>(u);
+      dst[kv_rank + 2 * i + 1] = from_f32<TC>(v);
+    } else {
+      dst[kv_rank + 2 * i] = from_f32<TC>(kr[2 * i]);
+      if (2 * i + 1 < rot_dim) dst[kv_rank + 2 * i + 1] = from_f32<TC>(kr[2 * i + 1]);
+    }
+  }
+}
+
+extern "C" int ts_latent_prepare(const float* proj, const float* q_norm, const float* kv_norm,
+                                 const float* freqs, void* cq, int out_type, void* pages,
+                                 int cache_type, const int* positions,
+                                 const int* entry_of_token, const int* table, int table_width,
+                                 int page_size, int num_tokens, int q_rank, int kv_rank,
+                                 int rot_dim, int rot_dims, float eps, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (q_rank <= 0 || kv_rank <= 0 || rot_dim < 0 || rot_dims % 2 || rot_dims > rot_dim ||
+      page_size <= 0 || table_width <= 0)
+    TS_FAIL("latent_prepare: bad sizes q_rank=%d kv_rank=%d rot_dim=%d rot_dims=%d", q_rank,
+            kv_rank, rot_dim, rot_dims);
+  TS_DISPATCH_TYPE(out_type, TO, TS_DISPATCH_TYPE(cache_type, TC,
+      hipLaunchKernelGGL((latent_prepare_kernel<TO, TC>), dim3(num_tokens), dim3(256), 0, stream,
+                         proj, q_norm, kv_norm, freqs, (TO*)cq, (TC*)pages, positions,
+                         entry_of_token, table, table_width, page_size, q_rank, kv_rank, rot_dim,
+                         rot_dims, eps)));
+  TS_CHECK_LAUNCH("latent_prepare");
+  return 0;
+}
+
+// ---------------------------------------------------------------- queries into the latent's space
+// q [T, heads, dim + rot_dim] float32; U_k [heads * dim, kv_rank].
+// out[t, h] = [ sum_d q[t, h, d] U_k[h * dim + d, :]  |  rot(q[t, h, dim:]) ], float32.
+// A workgroup serves one head and eight tokens, so a row of U_k is read once for eight.
+constexpr int kQueryTile = 8;
+
+template <typename TW>
+__global__ __launch_bounds__(256) void latent_query_kernel(
+    const float* __restrict__ q, const TW* __restrict__ uk, const float* __restrict__ freqs,
+    const int* __restrict__ positions, float* __restrict__ out, int num_tokens, int heads,
+    int dim, int rot_dim, int kv_rank, int rot_dims) {
+  extern __shared__ float q_s[];     // [kQueryTile][dim]
+  const int h = blockIdx.x, t0 = blockIdx.y * kQueryTile;
+  const int qd = dim + rot_dim, dl = kv_rank + rot_dim;
+  const int nt = min(kQueryTile, num_tokens - t0);
+  for (int i = threadIdx.x; i < kQueryTile * dim; i += blockDim.x) {
+    const int tt = i / dim, d = i % dim;
+    q_s[i] = tt < nt ? q[((int64_t)(t0 + tt) * heads + h) * qd + d] : 0.f;
+  }
+  __syncthreads();
+  const TW* w = uk + (int64_t)h * dim * kv_rank;
+  for (int r = threadIdx.x; r < kv_rank; r += blockDim.x) {
+    float acc[kQueryTile] = {};
+    for (int d = 0; d < dim; ++d) {
+      const float wv = to_f32(w[(int64_t)d * kv_rank + r]);
+#pragma unroll
+      for (int tt = 0; tt < kQueryTile; ++tt) acc[tt] = fmaf(q_s[tt * dim + d], wv, acc[tt]);
+    }
+#pragma unroll
+    for (int tt = 0; tt < kQueryTile; ++tt)
+      if (tt < nt) out[((int64_t)(t0 + tt) * heads + h) * dl + r] = acc[tt];
+  }
+  const int pairs = rot_dim / 2 + rot_dim % 2;
+  for (int i = threadIdx.x; i < nt * pairs; i += blockDim.x) {
+    const int tt = i / pairs, j = i % pairs;
+    const float* src = q + ((int64_t)(t0 + tt) * heads + h) * qd + dim;
+    float* dst = out + ((int64_t)(t0 + tt) * heads + h) * dl + kv_rank;
+    if (2 * j + 1 < rot_dims) {
+      rotate_pair(src[2 * j], src[2 * j + 1], positions[t0 + tt], freqs[j], &dst[2 * j],
+                  &dst[2 * j + 1]);
+    } else {
+      dst[2 * j] = src[2 * j];
+      if (2 * j + 1 < rot_dim) dst[2 * j + 1] = src[2 * j + 1];
+    }
+  }
+}
+
+extern "C" int ts_latent_query(const float* q, const void* uk, int weight_type,
+                               const float* freqs, const int* positions, float* out,
+                               int num_tokens, int heads, int dim, int rot_dim, int kv_rank,
+                               int rot_dims, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (heads <= 0 || dim <= 0 || kv_rank <= 0 || rot_dim < 0 || rot_dims % 2 || rot_dims > rot_dim)
+    TS_FAIL("latent_query: bad sizes heads=%d dim=%d rot_dim=%d kv_rank=%d", heads, dim, rot_dim,
+            kv_rank);
+  const size_t lds = (size_t)kQueryTile * dim * sizeof(float);
+  if (lds > 64 * 1024) TS_FAIL("latent_query: head size %d too large", dim);
+  const dim3 grid(heads, (num_tokens + kQueryTile - 1) / kQueryTile);
+  TS_DISPATCH_TYPE(weight_type, TW,
+                   hipLaunchKernelGGL(latent_query_kernel<TW>, grid, dim3(256), lds, stream, q,
+                                      (const TW*)uk, freqs, positions, out, num_tokens, heads, dim,
+                                      rot_dim, kv_rank, rot_dims));
+  TS_CHECK_LAUNCH("latent_query");
+  return 0;
+}
+
+// ---------------------------------------------------------------- attention
+// One wavefront per (token, head), four heads of a token to a workgroup (they read the same
+// rows).  Keys are cut into tiles of 64 starting at the first visible key, so the partition
+// and with it the rounding depends only on the token's position and the window.  In a
+// tile, lane j scores key j (a dot product over the whole row); then the lanes turn to the
+// columns of c and add the tile's weighted rows, key by key in order.
+constexpr int kMaxLatent = 1024;              // kv_rank + rot_dim
+constexpr int kLatentWaves = 4;
+constexpr int kMaxRankPerLane = 8;            // kv_rank <= 512
+
+template <typename TC>
+__global__ __launch_bounds__(kLatentWaves* kWave) void latent_attention_kernel(
+    const float* __restrict__ qa, const TC* __restrict__ pages, float* __restrict__ out,
+    const int* __restrict__ positions, const int* __restrict__ entry_of_token,
+    const int* __restrict__ table, int table_width, int page_size, int heads, int kv_rank,
+    int rot_dim, int window, float scale) {
+  extern __shared__ float lds[];      // per wave: q [dl], p [64], row numbers [64]
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int dl = kv_rank + rot_dim;
+  const int per_wave = dl + 2 * kWave;
+  float* q_s = lds + (size_t)wave * per_wave;
+  float* p_s = q_s + dl;
+  int* row_s = (int*)(p_s + kWave);
+  const int t = blockIdx.x;
+  const int h = blockIdx.y * kLatentWaves + wave;
+  if (h >= heads) return;             // waves are independent: no workgroup barrier below
+  const int pos = positions[t];
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int* tab = table + (int64_t)entry_of_token[t] * table_width;
+  const float* q = qa + ((int64_t)t * heads + h) * dl;
+  for (int d = lane; d < dl; d += kWave) q_s[d] = q[d];
+  __builtin_amdgcn_wave_barrier();
+  const bool by4 = dl % 4 == 0 && ((uintptr_t)pages & 15) == 0;
+
+  float m = -INFINITY, l = 0.f;
+  float acc[kMaxRankPerLane] = {};
+  for (int j0 = lo; j0 <= pos; j0 += kWave) {
+    const int j = j0 + lane;
+    float s = -INFINITY;
+    int row = -1;               // the token's row in the pages
+    if (j <= pos) {
+      const int page = tab[j / page_size];
+      if (page >= 0) {
+        row = page * page_size + j % page_size;
+        const TC* kr = pages + (int64_t)row * dl;
+        float dot = 0.f;
+        if (by4) {
+          for (int d = 0; d < dl; d += 4) {
+            const f32x4_l k4 = load4_l(kr + d);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dot = fmaf(q_s[d + e], k4[e], dot);
+          }
+        } else {
+          for (int d = 0; d < dl; ++d) dot = fmaf(q_s[d], to_f32(kr[d]), dot);
+        }
+        s = dot * scale;
+      }
+    }
+    const float m_new = fmaxf(m, wave_max(s));
+    const float corr = m_new == -INFINITY ? 1.f : expf(m - m_new);
+    const float p = (row >= 0 && m_new != -INFINITY) ? expf(s - m_new) : 0.f;
+    l = l * corr + wave_sum(p);
+    m = m_new;
+    p_s[lane] = p;
+    row_s[lane] = row;
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int r = 0; r < kMaxRankPerLane; ++r) acc[r] *= corr;
+    const int n = min(kWave, pos - j0 + 1);
+    for (int jj = 0; jj < n; ++jj) {
+      if (row_s[jj] < 0) continue;
+      const int64_t vr = (int64_t)row_s[jj] * dl;
+      const float pj = p_s[jj];
+#pragma unroll
+      for (int r = 0; r < kMaxRankPerLane; ++r) {
+        const int d = lane + r * kWave;
+        if (d < kv_rank) acc[r] = fmaf(pj, to_f32(pages[vr + d]), acc[r]);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  float* o = out + ((int64_t)t * heads + h) * kv_rank;
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+#pragma unroll
+  for (int r = 0; r < kMaxRankPerLane; ++r) {
+    const int d = lane + r * kWave;
+    if (d < kv_rank) o[d] = acc[r] * inv;
+  }
+}
+
+extern "C" int ts_latent_attention(const float* qa, const void* pages, int cache_type, float* out,
+                                   const int* positions, const int* entry_of_token,
+                                   const int* table, int table_width, int page_size,
+                                   int num_tokens, int heads, int kv_rank, int rot_dim,
+                                   int window, float scale, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  const int dl = kv_rank + rot_dim;
+  if (heads <= 0 || kv_rank <= 0 || rot_dim < 0 || page_size <= 0 || table_width <= 0)
+    TS_FAIL("latent_attention: bad sizes heads=%d kv_rank=%d rot_dim=%d", heads, kv_rank, rot_dim);
+  if (kv_rank > kMaxRankPerLane * kWave || dl > kMaxLatent)
+    TS_FAIL("latent_attention: latent of %d + %d elements, at most %d + %d are built", kv_rank,
+            rot_dim, kMaxRankPerLane * kWave, kMaxLatent - kMaxRankPerLane * kWave);
+  const size_t lds = (size_t)kLatentWaves * (dl + 2 * kWave) * sizeof(float);
+  const dim3 grid(num_tokens, (heads + kLatentWaves - 1) / kLatentWaves);
+  TS_DISPATCH_TYPE(cache_type, TC,
+                   hipLaunchKernelGGL(latent_attention_kernel<TC>, grid,
+                                      dim3(kLatentWaves * kWave), lds, stream, qa, (const TC*)pages,
+                                      out, positions, entry_of_token, table, table_width,
+                                      page_size, heads, kv_rank, rot_dim, window, scale));
+  TS_CHECK_LAUNCH("latent_attention");
+  return 0;
+}
+
+// ---------------------------------------------------------------- per-head product
+// x [T, heads, in] float32; W [heads * rows, in]; out[t, h, j] = sum_r W[h * rows + j, r]
+// x[t, h, r].  A workgroup serves one head and eight tokens; a wavefront takes a row of W,
+// its lanes stride over r, and the eight sums are added through the wavefront.
+template <typename TW, typename TO>
+__global__ __launch_bounds__(256) void head_linear_kernel(
+    const float* __restrict__ x, const TW* __restrict__ w, TO* __restrict__ out, int num_tokens,
+    int heads, int rows, int in) {
+  extern __shared__ float x_s[];      // [kQueryTile][in]
+  const int h = blockIdx.x, t0 = blockIdx.y * kQueryTile;
+  const int nt = min(kQueryTile, num_tokens - t0);
+  for (int i = threadIdx.x; i < kQueryTile * in; i += blockDim.x) {
+    const int tt = i / in, r = i % in;
+    x_s[i] = tt < nt ? x[((int64_t)(t0 + tt) * heads + h) * in + r] : 0.f;
+  }
+  __syncthreads();
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  for (int j = wave; j < rows; j += blockDim.x / kWave) {
+    const TW* wr = w + ((int64_t)h * rows + j) * in;
+    float acc[kQueryTile] = {};
+    for (int r = lane; r < in; r += kWave) {
+      const float wv = to_f32(wr[r]);
+#pragma unroll
+      for (int tt = 0; tt < kQueryTile; ++tt) acc[tt] = fmaf(x_s[tt * in + r], wv, acc[tt]);
+    }
+#pragma unroll
+    for (int tt = 0; tt < kQueryTile; ++tt) {
+      const float v = wave_sum(acc[tt]);
+      if (lane == 0 && tt < nt) out[((int64_t)(t0 + tt) * heads + h) * rows + j] = from_f32<TO>(v);
+    }
+  }
+}
+
+extern "C" int ts_head_linear(const float* x, const void* w, int weight_type, void* out,
+                              int out_type, int num_tokens, int heads, int rows, int in,
+                              hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (heads <= 0 || rows <= 0 || in <= 0) TS_FAIL("head_linear: bad sizes");
+  const size_t lds = (size_t)kQueryTile * in * sizeof(float);
+  if (lds > 64 * 1024) TS_FAIL("head_linear: rows of %d elements too long", in);
+  const dim3 grid(heads, (num_tokens + kQueryTile - 1) / kQueryTile);
+  TS_DISPATCH_TYPE(weight_type, TW, TS_DISPATCH_TYPE(out_type, TO,
+      hipLaunchKernelGGL((head_linear_kernel<TW, TO>), grid, dim3(256), lds, stream, x,
+                         (const TW*)w, (TO*)out, num_tokens, heads, rows, in)));
+  TS_CHECK_LAUNCH("head_linear");
+  return 0;
+}

@@ -1,0 +1,290 @@
+// Kernels of a selective state-space mixer with one scalar decay per head and token:
+// the short causal convolution with SiLU, the recurrence itself, and the gated group norm
+// behind it.  All arithmetic in float32; the recurrence's state and the convolution's last
+// inputs live in float32 per-request slots and are carried from step to step.
+//
+// A request's state is read only where a portion does not start at position 0, and is
+// written once a portion, by the thread that owns the element.
+#include "common.h"
+
+struct BatchView {
+  const int* positions;       // [T]
+  const int* entry_of_token;  // [T]
+  const int* q_start;         // [B + 1]
+  const int* slot_ids;        // [B]
+};
+
+__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
+__device__ __forceinline__ float softplus_f(float v) { return v > 20.f ? v : log1pf(expf(v)); }
+
+// ---------------------------------------------------------------- convolution
+// u = rows of `proj` (leading dimension ld) from column `col`, `channels` wide.
+// out_t[c] = silu(bias[c] + sum_k w[c][k] * u_(t - (taps-1) + k)[c]); inputs in front of
+// the sequence are zero, inputs in front of the portion come from state[slot][taps-1][C],
+// whose row j holds the input at position start - (taps-1) + j.
+
+// One thread per (token, channel); writes no state.
+__global__ __launch_bounds__(256) void conv_silu_kernel(
+    const float* __restrict__ proj, int ld, int col, int channels, int taps,
+    const float* __restrict__ w, const float* __restrict__ bias, const float* __restrict__ state,
+    float* __restrict__ out, BatchView b, int num_tokens) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)num_tokens * channels) return;
+  const int t = (int)(idx / channels), c = (int)(idx % channels);
+  const int e = b.entry_of_token[t];
+  const int first = b.q_start[e], pos = b.positions[t];
+  const float* st = state + (int64_t)b.slot_ids[e] * (taps - 1) * channels;
+  float acc = bias[c];
+  for (int k = 0; k < taps; ++k) {
+    const int back = taps - 1 - k;
+    if (pos - back < 0) continue;
+    float v;
+    if (t - back >= first) v = proj[(int64_t)(t - back) * ld + col + c];
+    else v = st[(int64_t)(taps - 1 - (first - (t - back))) * channels + c];
+    acc = fmaf(w[c * taps + k], v, acc);
+  }
+  out[(int64_t)t * channels + c] = silu_f(acc);
+}
+
+// One thread per (entry, channel): the state after the portion.  Row j takes the input at
+// position end - (taps-1) + j: from the portion, from the old state further up (read before
+// any row at or above it is written: j ascends), or zero in front of the sequence.
+__global__ __launch_bounds__(256) void conv_state_kernel(
+    const float* __restrict__ proj, int ld, int col, int channels, int taps,
+    float* __restrict__ state, BatchView b, int num_entries) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)num_entries * channels) return;
+  const int e = (int)(idx / channels), c = (int)(idx % channels);
+  const int first = b.q_start[e], n = b.q_start[e + 1] - first;
+  const int start = b.positions[first];
+  float* st = state + (int64_t)b.slot_ids[e] * (taps - 1) * channels;
+  for (int j = 0; j < taps - 1; ++j) {
+    const int p = start + n - (taps - 1) + j;
+    float v = 0.f;
+    if (p >= start) v = proj[(int64_t)(first + p - start) * ld + col + c];
+    else if (p >= 0) v = st[(int64_t)(j + n) * channels + c];
+    st[(int64_t)j * channels + c] = v;
+  }
+}
+
+// One thread per (entry, channel) walks the entry's tokens with the last inputs in
+// registers and leaves the state: one kernel for steps of few tokens per entry.
+constexpr int kMaxTapsInRegisters = 8;
+__global__ __launch_bounds__(256) void conv_silu_walk_kernel(
+    const float* __restrict__ proj, int ld, int col, int channels, int taps,
+    const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ state,
+    float* __restrict__ out, BatchView b, int num_entries) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)num_entries * channels) return;
+  const int e = (int)(idx / channels), c = (int)(idx % channels);
+  const int first = b.q_start[e], end = b.q_start[e + 1];
+  const int start = b.positions[first];
+  float* st = state + (int64_t)b.slot_ids[e] * (taps - 1) * channels;
+  float hist[kMaxTapsInRegisters], wk[kMaxTapsInRegisters];
+#pragma unroll
+  for (int j = 0; j < kMaxTapsInRegisters; ++j) {
+    hist[j] = 0.f;
+    wk[j] = j < taps ? w[c * taps + j] : 0.f;
+    // hist[j], j < taps-1: the input at position start - (taps-1) + j
+    if (j < taps - 1 && start - (taps - 1) + j >= 0) hist[j] = st[(int64_t)j * channels + c];
+  }
+  const float bc = bias[c];
+  for (int t = first; t < end; ++t) {
+    const float v = proj[(int64_t)t * ld + col + c];
+    float acc = bc;
+#pragma unroll
+    for (int k = 0; k < kMaxTapsInRegisters; ++k) {
+      if (k < taps - 1) acc = fmaf(wk[k], hist[k], acc);
+      else if (k == taps - 1) acc = fmaf(wk[k], v, acc);
+    }
+    out[(int64_t)t * channels + c] = silu_f(acc);
+#pragma unroll
+    for (int k = 0; k < kMaxTapsInRegisters - 1; ++k) {
+      if (k < taps - 2) hist[k] = hist[k + 1];
+      else if (k == taps - 2) hist[k] = v;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < kMaxTapsInRegisters; ++j)
+    if (j < taps - 1) st[(int64_t)j * channels + c] = hist[j];
+}
+
+extern "C" int ts_conv_silu(const float* proj, int ld, int col, int channels, int taps,
+                            const float* w, const float* bias, float* state, float* out,
+                            const int* positions, const int* entry_of_token, const int* q_start,
+                            const int* slot_ids, int num_tokens, int num_entries, int max_q_len,
+                            hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (channels <= 0 || taps < 1 || col < 0 || col + channels > ld)
+    TS_FAIL("conv_silu: bad sizes channels=%d taps=%d col=%d ld=%d", channels, taps, col, ld);
+  BatchView b{positions, entry_of_token, q_start, slot_ids};
+  if (max_q_len <= 4 && taps <= kMaxTapsInRegisters) {
+    const int64_t n = (int64_t)num_entries * channels;
+    hipLaunchKernelGGL(conv_silu_walk_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                       stream, proj, ld, col, channels, taps, w, bias, state, out, b,
+                       num_entries);
+    TS_CHECK_LAUNCH("conv_silu (walk)");
+    return 0;
+  }
+  const int64_t n = (int64_t)num_tokens * channels;
+  hipLaunchKernelGGL(conv_silu_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
+                     proj, ld, col, channels, taps, w, bias, state, out, b, num_tokens);
+  TS_CHECK_LAUNCH("conv_silu");
+  if (taps > 1) {
+    const int64_t m = (int64_t)num_entries * channels;
+    hipLaunchKernelGGL(conv_state_kernel, dim3((unsigned)((m + 255) / 256)), dim3(256), 0, stream,
+                       proj, ld, col, channels, taps, state, b, num_entries);
+    TS_CHECK_LAUNCH("conv_state");
+  }
+  return 0;
+}
+
+// ---------------------------------------------------------------- recurrence
+// Per head h (group g): d = softplus(dt + dt_bias[h]), a = exp(-exp(A_log[h]) d),
+//   S <- a S + (d B_g) x_h^T   (S: N x P),   y_h = S^T C_g + D[h] x_h.
+// A workgroup serves one (entry, head, 32 columns of P): thread (p, s) keeps rows
+// s, s + 8, ... of column p in registers, walks the entry's tokens in order and adds the
+// eight slices of a column's dot product through the wavefront.  The operands of the next
+// token are fetched while the current one is computed.
+struct ScanArgs {
+  const float* xbc;       // [T, channels]: x (heads*P) | B (groups*N) | C (groups*N)
+  const float* proj;      // [T, ld]: dt at column dt_col
+  const float* dt_bias;   // [heads]
+  const float* a_log;     // [heads]
+  const float* d_skip;    // [heads]
+  float* state;           // [slots, heads, N, P]
+  float* y;               // [T, heads*P]
+  BatchView b;
+  int ld, dt_col, channels, heads, P, N, groups;
+};
+
+constexpr int kScanSlices = 8;
+constexpr int kScanCols = 32;
+
+template <int NI>
+__global__ __launch_bounds__(kScanSlices* kScanCols) void ssm_scan_kernel(ScanArgs a) {
+  const int h = blockIdx.x, e = blockIdx.y;
+  const int p = blockIdx.z * kScanCols + threadIdx.x / kScanSlices;
+  const int s = threadIdx.x % kScanSlices;
+  const bool live = p < a.P;
+  const int pc = live ? p : a.P - 1;      // idle columns shadow the last one and store nothing
+  const int g = h / (a.heads / a.groups);
+  const int first = a.b.q_start[e], end = a.b.q_start[e + 1];
+  const int inner = a.heads * a.P;
+  const int N = a.N;
+  float* st = a.state + ((int64_t)a.b.slot_ids[e] * a.heads + h) * N * a.P;
+  float S[NI];
+  const bool fresh = a.b.positions[first] == 0;
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+    const int n = s + kScanSlices * i;
+    S[i] = (!fresh && n < N) ? st[(int64_t)n * a.P + pc] : 0.f;
+  }
+  const float decay_rate = -expf(a.a_log[h]);
+  const float bias = a.dt_bias[h], skip = a.d_skip[h];
+  const int b_col = inner + g * N, c_col = inner + a.groups * N + g * N;
+
+  float nB[NI], nC[NI], nx, ndt;
+  auto fetch = [&](int t) {
+    const float* row = a.xbc + (int64_t)t * a.channels;
+    nx = row[h * a.P + pc];
+    ndt = a.proj[(int64_t)t * a.ld + a.dt_col + h];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int n = s + kScanSlices * i;
+      nB[i] = n < N ? row[b_col + n] : 0.f;
+      nC[i] = n < N ? row[c_col + n] : 0.f;
+    }
+  };
+  if (first < end) fetch(first);
+  for (int t = first; t < end; ++t) {
+    float B[NI], C[NI];
+    const float x = nx, dt_raw = ndt;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) { B[i] = nB[i]; C[i] = nC[i]; }
+    if (t + 1 < end) fetch(t + 1);
+    const float d = softplus_f(dt_raw + bias);
+    const float decay = expf(decay_rate * d);
+    const float dx = d * x;
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      S[i] = fmaf(decay, S[i], B[i] * dx);
+      acc = fmaf(S[i], C[i], acc);
+    }
+    acc += __shfl_xor(acc, 1, kWave);
+    acc += __shfl_xor(acc, 2, kWave);
+    acc += __shfl_xor(acc, 4, kWave);
+    if (s == 0 && live) a.y[(int64_t)t * inner + h * a.P + p] = fmaf(skip, x, acc);
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int n = s + kScanSlices * i;
+      if (n < N) st[(int64_t)n * a.P + p] = S[i];
+    }
+  }
+}
+
+extern "C" int ts_ssm_scan(const float* xbc, const float* proj, int ld, int dt_col,
+                           const float* dt_bias, const float* a_log, const float* d_skip,
+                           float* state, float* y, const int* positions,
+                           const int* entry_of_token, const int* q_start, const int* slot_ids,
+                           int num_tokens, int num_entries, int heads, int P, int N, int groups,
+                           hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (heads <= 0 || P <= 0 || N <= 0 || groups <= 0 || heads % groups)
+    TS_FAIL("ssm_scan: bad sizes heads=%d vdim=%d state=%d groups=%d", heads, P, N, groups);
+  if (N > kScanSlices * 32) TS_FAIL("ssm_scan: state of %d rows, at most %d are built", N, kScanSlices * 32);
+  if (dt_col < 0 || dt_col + heads > ld) TS_FAIL("ssm_scan: dt columns outside the projection");
+  ScanArgs a{xbc, proj, dt_bias, a_log, d_skip, state, y,
+             BatchView{positions, entry_of_token, q_start, slot_ids},
+             ld, dt_col, heads * P + 2 * groups * N, heads, P, N, groups};
+  const dim3 grid(heads, num_entries, (P + kScanCols - 1) / kScanCols);
+  const dim3 block(kScanSlices * kScanCols);
+  const int ni = (N + kScanSlices - 1) / kScanSlices;
+  if (ni <= 2) hipLaunchKernelGGL(ssm_scan_kernel<2>, grid, block, 0, stream, a);
+  else if (ni <= 4) hipLaunchKernelGGL(ssm_scan_kernel<4>, grid, block, 0, stream, a);
+  else if (ni <= 8) hipLaunchKernelGGL(ssm_scan_kernel<8>, grid, block, 0, stream, a);
+  else if (ni <= 16) hipLaunchKernelGGL(ssm_scan_kernel<16>, grid, block, 0, stream, a);
+  else hipLaunchKernelGGL(ssm_scan_kernel<32>, grid, block, 0, stream, a);
+  TS_CHECK_LAUNCH("ssm_scan");
+  return 0;
+}
+
+// ---------------------------------------------------------------- gate and group norm
+// v = y * silu(z) (z: the first `inner` columns of proj); each of `groups` equal parts of
+// a row is divided by its own root mean square; out = that * w.
+template <typename TO>
+__global__ __launch_bounds__(256) void gated_group_norm_kernel(
+    const float* __restrict__ y, const float* __restrict__ proj, int ld,
+    const float* __restrict__ w, TO* __restrict__ out, int inner, int groups, float eps) {
+  __shared__ float scratch[16];
+  const int64_t t = blockIdx.x;
+  const int grp = blockIdx.y, size = inner / groups;
+  const float* yr = y + t * inner + grp * size;
+  const float* zr = proj + t * ld + grp * size;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < size; i += blockDim.x) {
+    const float v = yr[i] * silu_f(zr[i]);
+    ss += v * v;
+  }
+  const float r = 1.0f / sqrtf(block_sum(ss, scratch) / (float)size + eps);
+  TO* o = out + t * inner + grp * size;
+  const float* wr = w + grp * size;
+  for (int i = threadIdx.x; i < size; i += blockDim.x)
+    o[i] = from_f32<TO>(yr[i] * silu_f(zr[i]) * r * wr[i]);
+}
+
+extern "C" int ts_gated_group_norm(const float* y, const float* proj, int ld, const float* w,
+                                   void* out, int out_type, int rows, int inner, int groups,
+                                   float eps, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (inner <= 0 || groups <= 0 || inner % groups || inner > ld)
+    TS_FAIL("gated_group_norm: bad sizes inner=%d groups=%d ld=%d", inner, groups, ld);
+  TS_DISPATCH_TYPE(out_type, TO,
+                   hipLaunchKernelGGL(gated_group_norm_kernel<TO>, dim3(rows, groups), dim3(256),
+                                      0, stream, y, proj, ld, w, (TO*)out, inner, groups, eps));
+  TS_CHECK_LAUNCH("gated_group_norm");
+  return 0;
+}

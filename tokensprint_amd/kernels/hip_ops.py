@@ -930,3 +930,230 @@ class HipOps:
         self._call(self.lib.ts_sample, _ptr(logits), _ptr(temperatures), _ptr(keys), _ptr(out),
                    _ptr(part_v), _ptr(part_i), R, logits.shape[1], self._stream())
         return out
+
+    # ------------------------------------------------------------ sandwich-norm rows
+    def _batch_ptrs(self, batch, T):
+        self._check("positions", batch.positions, torch.int32, shape=(T,))
+        self._check("entry_of_token", batch.entry_of_token, torch.int32, shape=(T,))
+        self._check("q_start", batch.q_start, torch.int32, shape=(batch.num_entries + 1,))
+        self._check("slot_ids", batch.slot_ids, torch.int32, shape=(batch.num_entries,))
+        if T != batch.num_tokens:
+            raise ValueError(f"{T} rows for a batch of {batch.num_tokens} tokens")
+        return (_ptr(batch.positions), _ptr(batch.entry_of_token), _ptr(batch.q_start),
+                _ptr(batch.slot_ids))
+
+    def _check_state(self, name, state, shape, dtype=torch.float32):
+        self._check(name, state, dtype, ndim=len(shape) + 1)
+        if tuple(state.shape[1:]) != tuple(shape):
+            raise ValueError(f"{name}: shape {tuple(state.shape)}, expected [slots, "
+                             f"{', '.join(str(s) for s in shape)}]")
+
+    def bigram_embed(self, table, bigram, norm_w, batch, prev_state, *, scale, buckets,
+                     mul_prev, mul_cur, eps):
+        """norm(table[id] * scale + bigram[row]) -> float32 [T, width]; row hashes the
+        previous and the current token (`prev_state` [slots, 1] int32 keeps a request's
+        last token between steps), the last row serves a sequence's first token."""
+        self._check("embedding table", table, self._FLOATS, ndim=2)
+        W = table.shape[1]
+        self._check("bigram table", bigram, table.dtype, shape=(buckets + 1, W))
+        self._check("norm weight", norm_w, torch.float32, shape=(W,))
+        self._check("token ids", batch.token_ids, torch.int32, ndim=1)
+        T = batch.token_ids.shape[0]
+        pos, eot, qs, slots = self._batch_ptrs(batch, T)
+        self._check_state("previous tokens", prev_state, (1,), torch.int32)
+        out = torch.empty(T, W, dtype=torch.float32, device=self.device)
+        self._call(self.lib.ts_bigram_embed, _ptr(table), _ptr(bigram), _TYPE_CODE[table.dtype],
+                   _ptr(norm_w), _ptr(batch.token_ids), pos, eot, qs, slots, _ptr(prev_state),
+                   _ptr(out), T, W, c_float(scale), int(buckets), int(mul_prev), int(mul_cur),
+                   c_float(eps), self._stream())
+        return out
+
+    def postnorm_add(self, resid, delta, post_w, eps):
+        """resid += delta / rms(delta) * post_w, in place (float32)."""
+        self._postnorm(resid, delta, post_w, eps, None, 0.0, None)
+
+    def postnorm_add_norm(self, resid, delta, post_w, post_eps, norm_w, norm_eps, out_dtype):
+        """The same, and the norm (norm_w, norm_eps) of the new resid in `out_dtype`."""
+        return self._postnorm(resid, delta, post_w, post_eps, norm_w, norm_eps, out_dtype)
+
+    def _postnorm(self, resid, delta, post_w, post_eps, norm_w, norm_eps, out_dtype):
+        delta = self._rows(delta)
+        self._check("resid", resid, torch.float32, ndim=2)
+        self._check("delta", delta, torch.float32, shape=resid.shape)
+        W = resid.shape[1]
+        self._check("post-norm weight", post_w, torch.float32, shape=(W,))
+        out = None
+        if norm_w is not None:
+            self._check("norm weight", norm_w, torch.float32, shape=(W,))
+            out = torch.empty(resid.shape, dtype=out_dtype, device=self.device)
+        self._call(self.lib.ts_postnorm_add, _ptr(resid), _ptr(delta), _ptr(post_w),
+                   c_float(post_eps), _ptr(norm_w), c_float(norm_eps), _ptr(out),
+                   _TYPE_CODE[out_dtype] if out is not None else 0, resid.shape[0], W,
+                   self._stream())
+        return out
+
+    def norm_token_shift(self, resid, norm_w, eps, shift_w, batch, state, out_dtype):
+        """h = norm(resid); out_t = h_t + (h_(t-1) - h_t) * shift_w.  `state` [slots, width]
+        float32 carries a request's last h from step to step."""
+        self._check("resid", resid, torch.float32, ndim=2)
+        T, W = resid.shape
+        self._check("norm weight", norm_w, torch.float32, shape=(W,))
+        self._check("shift weight", shift_w, torch.float32, shape=(W,))
+        self._check_state("shift state", state, (W,))
+        pos, eot, qs, slots = self._batch_ptrs(batch, T)
+        out = torch.empty(T, W, dtype=out_dtype, device=self.device)
+        self._call(self.lib.ts_norm_token_shift, _ptr(resid), _ptr(norm_w), c_float(eps),
+                   _ptr(shift_w), _ptr(state), _ptr(out), _TYPE_CODE[out_dtype], pos, eot, qs,
+                   slots, T, W, self._stream())
+        return out
+
+    def polynorm(self, z, coef, eps, out_dtype):
+        """a N(z) + b N(z^2) + c N(z^3) + e with N(v) = v / rms(v) per row; coef = (a, b, c, e)."""
+        self._check("z", z, torch.float32, ndim=2)
+        self._check("coefficients", coef, torch.float32, shape=(4,))
+        out = torch.empty(z.shape, dtype=out_dtype, device=self.device)
+        self._call(self.lib.ts_polynorm, _ptr(z), _ptr(coef), _ptr(out), _TYPE_CODE[out_dtype],
+                   z.shape[0], z.shape[1], c_float(eps), self._stream())
+        return out
+
+    # ------------------------------------------------------------ state-space mixer
+    def conv_silu(self, proj, col, channels, weight, bias, batch, state):
+        """Causal convolution per channel over columns [col, col + channels) of `proj`
+        (float32 [T, ld]), bias, SiLU -> float32 [T, channels].  weight [channels, taps]
+        (the last tap is the current token's); `state` [slots, taps - 1, channels] carries
+        a request's last inputs."""
+        self._check("proj", proj, torch.float32, ndim=2)
+        T, ld = proj.shape
+        self._check("conv weight", weight, torch.float32, ndim=2)
+        taps = weight.shape[1]
+        if weight.shape[0] != channels or col < 0 or col + channels > ld:
+            raise ValueError(f"conv_silu: {channels} channels from column {col} of {ld}, "
+                             f"weight {tuple(weight.shape)}")
+        self._check("conv bias", bias, torch.float32, shape=(channels,))
+        self._check_state("conv state", state, (taps - 1, channels))
+        pos, eot, qs, slots = self._batch_ptrs(batch, T)
+        out = torch.empty(T, channels, dtype=torch.float32, device=self.device)
+        self._call(self.lib.ts_conv_silu, _ptr(proj), ld, col, channels, taps, _ptr(weight),
+                   _ptr(bias), _ptr(state), _ptr(out), pos, eot, qs, slots, T,
+                   batch.num_entries, int(batch.max_q_len), self._stream())
+        return out
+
+    def ssm_scan(self, xbc, proj, dt_col, dt_bias, a_log, d_skip, batch, state, *, heads, vdim,
+                 state_rows, groups):
+        """The recurrence S <- exp(-exp(A_log) d) S + d B x^T, y = S^T C + D x per head,
+        d = softplus(dt + dt_bias), over each entry's tokens in order -> float32
+        [T, heads * vdim].  xbc [T, heads*vdim + 2*groups*state_rows]; dt is `heads`
+        columns of `proj` from `dt_col`; `state` [slots, heads, state_rows, vdim]."""
+        inner, N = heads * vdim, state_rows
+        self._check("xbc", xbc, torch.float32, ndim=2)
+        T = xbc.shape[0]
+        if xbc.shape[1] != inner + 2 * groups * N:
+            raise ValueError(f"ssm_scan: xbc has {xbc.shape[1]} columns, expected "
+                             f"{inner + 2 * groups * N}")
+        self._check("proj", proj, torch.float32, ndim=2)
+        if proj.shape[0] != T or dt_col < 0 or dt_col + heads > proj.shape[1]:
+            raise ValueError("ssm_scan: dt columns outside the projection")
+        for name, v in (("dt_bias", dt_bias), ("A_log", a_log), ("D", d_skip)):
+            self._check(name, v, torch.float32, shape=(heads,))
+        self._check_state("recurrent state", state, (heads, N, vdim))
+        pos, eot, qs, slots = self._batch_ptrs(batch, T)
+        y = torch.empty(T, inner, dtype=torch.float32, device=self.device)
+        self._call(self.lib.ts_ssm_scan, _ptr(xbc), _ptr(proj), proj.shape[1], dt_col,
+                   _ptr(dt_bias), _ptr(a_log), _ptr(d_skip), _ptr(state), _ptr(y), pos, eot, qs,
+                   slots, T, batch.num_entries, heads, vdim, N, groups, self._stream())
+        return y
+
+    def gated_group_norm(self, y, proj, norm_w, groups, eps, out_dtype):
+        """(y * silu(z)) normalised in `groups` equal parts, times norm_w; z is the first
+        y.shape[1] columns of `proj`."""
+        self._check("y", y, torch.float32, ndim=2)
+        T, inner = y.shape
+        self._check("proj", proj, torch.float32, ndim=2)
+        if proj.shape[0] != T or proj.shape[1] < inner or inner % groups:
+            raise ValueError("gated_group_norm: shapes do not fit")
+        self._check("norm weight", norm_w, torch.float32, shape=(inner,))
+        out = torch.empty(T, inner, dtype=out_dtype, device=self.device)
+        self._call(self.lib.ts_gated_group_norm, _ptr(y), _ptr(proj), proj.shape[1], _ptr(norm_w),
+                   _ptr(out), _TYPE_CODE[out_dtype], T, inner, groups, c_float(eps),
+                   self._stream())
+        return out
+
+    # ------------------------------------------------------------ latent attention
+    def _check_latent(self, cache, table, batch, dl):
+        self._check("latent pages", cache.k_pages, self._FLOATS,
+                    shape=(cache.num_pages, cache.page_size, dl))
+        self._check("block table", table, torch.int32, ndim=2)
+        if table.shape[0] != batch.num_entries:
+            raise ValueError("block table rows differ from the batch's entries")
+
+    def latent_prepare(self, proj, batch, table, cache, *, q_rank, kv_rank, rot_dim, q_norm,
+                       kv_norm, eps, freqs, rot_dims, out_dtype):
+        """Rows [q latent | kv latent | shared key part] (float32): the normalised q latent
+        comes back in `out_dtype`; the normalised kv latent and the rotated key part are
+        written to the tokens' rows of the latent pages."""
+        self._check("proj", proj, torch.float32, ndim=2)
+        T = proj.shape[0]
+        dl = kv_rank + rot_dim
+        if proj.shape[1] != q_rank + dl:
+            raise ValueError(f"latent_prepare: rows of {proj.shape[1]}, expected {q_rank + dl}")
+        self._check("q norm", q_norm, torch.float32, shape=(q_rank,))
+        self._check("kv norm", kv_norm, torch.float32, shape=(kv_rank,))
+        self._check("frequencies", freqs, torch.float32, shape=(rot_dims // 2,))
+        self._check_latent(cache, table, batch, dl)
+        pos, eot, _, _ = self._batch_ptrs(batch, T)
+        cq = torch.empty(T, q_rank, dtype=out_dtype, device=self.device)
+        self._call(self.lib.ts_latent_prepare, _ptr(proj), _ptr(q_norm), _ptr(kv_norm),
+                   _ptr(freqs), _ptr(cq), _TYPE_CODE[out_dtype], _ptr(cache.k_pages),
+                   _TYPE_CODE[cache.k_pages.dtype], pos, eot, _ptr(table), table.shape[1],
+                   cache.page_size, T, q_rank, kv_rank, rot_dim, rot_dims, c_float(eps),
+                   self._stream())
+        return cq
+
+    def latent_query(self, q, w_uk, batch, *, heads, dim, rot_dim, kv_rank, freqs, rot_dims):
+        """q [T, heads*(dim+rot_dim)] float32 -> [T, heads, kv_rank+rot_dim] float32: the
+        unrotated part carried through U_k (w_uk [heads*dim, kv_rank]) into the latent's
+        space, the rotated part rotated at the token's position."""
+        self._check("q", q, torch.float32, ndim=2)
+        T = q.shape[0]
+        if q.shape[1] != heads * (dim + rot_dim):
+            raise ValueError("latent_query: q rows do not fit heads * (dim + rot_dim)")
+        self._check("U_k", w_uk, self._FLOATS, shape=(heads * dim, kv_rank))
+        self._check("frequencies", freqs, torch.float32, shape=(rot_dims // 2,))
+        self._check("positions", batch.positions, torch.int32, shape=(T,))
+        out = torch.empty(T, heads, kv_rank + rot_dim, dtype=torch.float32, device=self.device)
+        self._call(self.lib.ts_latent_query, _ptr(q), _ptr(w_uk), _TYPE_CODE[w_uk.dtype],
+                   _ptr(freqs), _ptr(batch.positions), _ptr(out), T, heads, dim, rot_dim, kv_rank,
+                   rot_dims, self._stream())
+        return out
+
+    def latent_attention(self, qa, batch, table, cache, *, heads, kv_rank, rot_dim, scale,
+                         window):
+        """Softmax attention of qa [T, heads, kv_rank+rot_dim] (float32) over the latent
+        pages -> sum_t p_t c_t, float32 [T, heads, kv_rank]."""
+        dl = kv_rank + rot_dim
+        self._check("qa", qa, torch.float32, ndim=3)
+        T = qa.shape[0]
+        if tuple(qa.shape[1:]) != (heads, dl):
+            raise ValueError("latent_attention: query shape does not fit")
+        self._check_latent(cache, table, batch, dl)
+        pos, eot, _, _ = self._batch_ptrs(batch, T)
+        out = torch.empty(T, heads, kv_rank, dtype=torch.float32, device=self.device)
+        self._call(self.lib.ts_latent_attention, _ptr(qa), _ptr(cache.k_pages),
+                   _TYPE_CODE[cache.k_pages.dtype], _ptr(out), pos, eot, _ptr(table),
+                   table.shape[1], cache.page_size, T, heads, kv_rank, rot_dim,
+                   int(window) if window else 0, c_float(scale), self._stream())
+        return out
+
+    def head_linear(self, x, weight, heads, out_dtype):
+        """x [T, heads, in] float32, weight [heads*rows, in] -> [T, heads*rows]: each head's
+        rows of the weight applied to that head's vector."""
+        self._check("x", x, torch.float32, ndim=3)
+        T, H, n_in = x.shape
+        self._check("weight", weight, self._FLOATS, ndim=2)
+        if H != heads or weight.shape[1] != n_in or weight.shape[0] % heads:
+            raise ValueError("head_linear: shapes do not fit")
+        rows = weight.shape[0] // heads
+        out = torch.empty(T, heads * rows, dtype=out_dtype, device=self.device)
+        self._call(self.lib.ts_head_linear, _ptr(x), _ptr(weight), _TYPE_CODE[weight.dtype],
+                   _ptr(out), _TYPE_CODE[out_dtype], T, heads, rows, n_in, self._stream())
+        return out

@@ -71,9 +71,14 @@ class Model:
 
     # ------------------------------------------------------------ caches
     def cache_needs(self):
-        """Per run: the cache need of its block, or None if the run owns no cache."""
-        return [self.blocks[run.layer].cache_need() if run.cache_of is None else None
-                for run in self.order]
+        """Per run: the cache need of its block, or None if the run owns no cache.  If the
+        embedding keeps state per request, its need follows as one more entry (the cache
+        view behind the last run's is the embedding's)."""
+        needs = [self.blocks[run.layer].cache_need() if run.cache_of is None else None
+                 for run in self.order]
+        if self.embedding.cache_need() is not None:
+            needs.append(self.embedding.cache_need())
+        return needs
 
     # ------------------------------------------------------------ step
     def forward(self, batch, caches) -> torch.Tensor:
@@ -82,7 +87,8 @@ class Model:
         `caches[r]` is the cache view owned by run r (None if it owns none).
         """
         ops = self.ctx.ops
-        resid = self.embedding.forward(batch.token_ids)
+        resid = self.embedding.forward_step(
+            batch, caches[len(self.order)] if len(caches) > len(self.order) else None)
         delta = None
         for r, run in enumerate(self.order):
             owner = r if run.cache_of is None else run.cache_of

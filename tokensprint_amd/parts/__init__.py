@@ -1,13 +1,14 @@
-from tokensprint_amd.parts import attention, block, feed_forward, norm, position  # noqa: F401
+from tokensprint_amd.parts import (attention, block, feed_forward, latent_attention, mamba2,  # noqa: F401
+                                   norm, position)
 from tokensprint_amd.parts.base import (
-    BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITIONS, Block, BuildContext,
-    FeedForward, Mixer, Norm, OutputHead, PagedKVNeed, Part, PositionEncoding, SlotStateNeed,
-    TensorDecl, TokenEmbedding, build_part, register,
+    BLOCKS, EMBEDDINGS, FEED_FORWARDS, FILTERS, HEADS, MIXERS, NORMS, POSITIONS, Block,
+    BuildContext, FeedForward, Mixer, Norm, OutputHead, PagedKVNeed, PagedLatentNeed, Part,
+    PositionEncoding, SlotStateNeed, StreamFilter, TensorDecl, TokenEmbedding, build_part, register,
 )
 from tokensprint_amd.parts.ends import Embedding, Head
 
 __all__ = [
-    "BLOCKS", "EMBEDDINGS", "FEED_FORWARDS", "HEADS", "MIXERS", "NORMS", "POSITIONS", "Block",
+    "BLOCKS", "EMBEDDINGS", "FILTERS", "PagedLatentNeed", "StreamFilter", "FEED_FORWARDS", "HEADS", "MIXERS", "NORMS", "POSITIONS", "Block",
     "BuildContext", "FeedForward", "Mixer", "Norm", "OutputHead", "PagedKVNeed", "Part",
     "PositionEncoding", "SlotStateNeed", "TensorDecl", "TokenEmbedding", "build_part",
     "register", "Embedding", "Head",

@@ -7,7 +7,8 @@ the step's batch description and, for a mixer, the cache of the run it executes.
 No part knows which model it is in.
 
 Registries map a `kind` string to a class, one registry per role:
-`MIXERS`, `FEED_FORWARDS`, `NORMS`, `POSITIONS`, `BLOCKS`, `EMBEDDINGS`, `HEADS`.  A test
+`MIXERS`, `FEED_FORWARDS`, `NORMS`, `POSITIONS`, `BLOCKS`, `EMBEDDINGS`, `HEADS`,
+`FILTERS`.  A test
 or a new architecture adds a part with `register(MIXERS, "my_kind")(MyClass)`.
 """
 
@@ -34,6 +35,10 @@ class TensorDecl:
     shape: tuple[int, ...]
     role: str = "matrix"
     optional: bool = False      # may be absent from the file (e.g. a tied head's copy)
+    #: (low, high) of the uniform draw random-weights mode makes for this tensor instead of
+    #: its role's rule (a decay's logarithm, a step's bias: values whose useful range is not
+    #: a norm weight's)
+    init: tuple[float, float] | None = None
 
 
 @dataclass(frozen=True)
@@ -46,11 +51,33 @@ class PagedKVNeed:
 
 
 @dataclass(frozen=True)
+class PagedLatentNeed:
+    """One vector of `dim` elements per token, in pages: what attention over a shared
+    latent keeps (every head reads the same vector as key and, in part, as value).
+    window None = every earlier token."""
+
+    dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
 class SlotStateNeed:
-    """A fixed-size per-request state tensor (shape without the slot axis)."""
+    """A fixed-size per-request state tensor (shape without the slot axis).  A run that
+    keeps several gives each a `name`; its cache view holds them as `states[name]`."""
 
     shape: tuple[int, ...]
     dtype: torch.dtype = torch.float32
+    name: str = "state"
+
+
+def flat_needs(need) -> tuple:
+    """A cache need as a tuple of single needs: None is empty, a single need is itself, a
+    tuple or list (a run that keeps pages and state, or several states) is flattened."""
+    if need is None:
+        return ()
+    if isinstance(need, (tuple, list)):
+        return tuple(n for item in need for n in flat_needs(item))
+    return (need,)
 
 
 @dataclass
@@ -126,7 +153,9 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    def cache_need(self) -> PagedKVNeed | SlotStateNeed | None:
+    def cache_need(self):
+        """What a run of this mixer keeps per request: None, a PagedKVNeed, a
+        PagedLatentNeed, a SlotStateNeed, or a tuple of them (at most one paged need)."""
         return None
 
     def forward(self, h: torch.Tensor, batch, cache, write_cache: bool) -> torch.Tensor:
@@ -164,12 +193,34 @@ class FeedForward(Part):
         return self.forward(h, batch), resid
 
 
+class StreamFilter(Part):
+    """Applied by a block to what its mixer reads, behind the mixer's norm: h [T, width]
+    float32 -> the mixer's input in the activation dtype.  It may keep per-request state
+    (`cache_need`, as a mixer's) in the cache view of the run it executes."""
+
+    def cache_need(self):
+        return None
+
+    def forward_from_stream(self, resid: torch.Tensor, norm: "Norm", batch, cache) -> torch.Tensor:
+        """The filtered norm of the rows of the stream."""
+        raise NotImplementedError
+
+
 class TokenEmbedding(Part):
     """The model's first part: token ids (int32 [T]) -> the residual stream, float32
     [T, width]."""
 
+    def cache_need(self):
+        """Per-request state of the embedding (as a mixer's `cache_need`), or None."""
+        return None
+
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
+
+    def forward_step(self, batch, cache) -> torch.Tensor:
+        """The stream of the step's tokens; `cache` is the embedding's own cache view (None
+        unless `cache_need` asks for one).  Default: a function of the token ids alone."""
+        return self.forward(batch.token_ids)
 
 
 class OutputHead(Part):
@@ -213,9 +264,14 @@ class Block:
         return [getattr(self, role) for role in self.ROLES if getattr(self, role) is not None]
 
     def cache_need(self):
-        """What a run of this block keeps per request: its mixer's need, if it has one."""
-        mixer = getattr(self, "mixer", None)
-        return mixer.cache_need() if mixer is not None else None
+        """What a run of this block keeps per request: the needs of its parts that have
+        one (the mixer, a filter in front of it)."""
+        needs = ()
+        for part in self.parts():
+            probe = getattr(part, "cache_need", None)
+            if callable(probe):
+                needs += flat_needs(probe())
+        return needs[0] if len(needs) == 1 else (needs or None)
 
     def entry_hint(self):
         """The `stream_hint` of the part of this block that reads the stream first."""
@@ -235,6 +291,7 @@ POSITIONS: dict[str, type] = {}
 BLOCKS: dict[str, type] = {}
 EMBEDDINGS: dict[str, type] = {}
 HEADS: dict[str, type] = {}
+FILTERS: dict[str, type] = {}
 
 
 def register(registry: dict[str, type], kind: str, *, replace: bool = False):

@@ -11,7 +11,7 @@ from __future__ import annotations
 import torch
 
 from tokensprint_amd.kernels.stream import fused_rmsnorm_of
-from tokensprint_amd.parts.base import (EMBEDDINGS, HEADS, OutputHead, TensorDecl,
+from tokensprint_amd.parts.base import (EMBEDDINGS, HEADS, OutputHead, SlotStateNeed, TensorDecl,
                                         TokenEmbedding, register)
 
 
@@ -36,6 +36,54 @@ class Embedding(TokenEmbedding):
 
     def step_read_tensors(self):
         return []          # a step reads the rows of its tokens, not the table
+
+
+@register(EMBEDDINGS, "bigram_embedding")
+class BigramEmbedding(TokenEmbedding):
+    """x[t] = norm(E[id_t] * scale + G[row_t]): a second table G is indexed by a hash of
+    the previous and the current token, row_t = (id_(t-1) * mul_prev + id_t * mul_cur) mod
+    buckets, and by its last row (index `buckets`) for a sequence's first token; the sum
+    passes an RMS norm.  A request's last token is kept in its state slot, so a step's
+    first token finds its predecessor whatever step brought it.
+
+    params: weight, bigram, norm (tensor names), vocab_size, scale, buckets, mul_prev,
+    mul_cur, eps."""
+
+    def __init__(self, params, ctx):
+        super().__init__(params, ctx)
+        p = params
+        self.name, self.bigram_name, self.norm_name = p["weight"], p["bigram"], p["norm"]
+        self.vocab, self.buckets = int(p["vocab_size"]), int(p["buckets"])
+        self.scale, self.eps = float(p["scale"]), float(p["eps"])
+        self.mul_prev, self.mul_cur = int(p["mul_prev"]), int(p["mul_cur"])
+        self.table = self.bigram = self.norm_w = None
+
+    def tensors(self):
+        W = self.ctx.width
+        return {self.name: TensorDecl((self.vocab, W)),
+                self.bigram_name: TensorDecl((self.buckets + 1, W)),
+                self.norm_name: TensorDecl((W,), role="vector")}
+
+    def load(self, get):
+        self.table, self.bigram = get(self.name), get(self.bigram_name)
+        self.norm_w = get(self.norm_name)
+
+    def cache_need(self):
+        return SlotStateNeed((1,), torch.int32, "prev_token")
+
+    def forward(self, token_ids):
+        raise RuntimeError("a bigram embedding needs the step's batch: use forward_step")
+
+    def forward_step(self, batch, cache):
+        if cache is None or "prev_token" not in cache.states:
+            raise RuntimeError("bigram_embedding needs its per-request state")
+        return self.ops.bigram_embed(
+            self.table, self.bigram, self.norm_w, batch, cache.states["prev_token"],
+            scale=self.scale, buckets=self.buckets, mul_prev=self.mul_prev,
+            mul_cur=self.mul_cur, eps=self.eps)
+
+    def step_read_tensors(self):
+        return [self.norm_w]
 
 
 @register(HEADS, "head")

@@ -40,3 +40,34 @@ class RotaryEncoding(PositionEncoding):
         self.ops.rope_inplace(q, positions, self.cos, self.sin)
         if k is not None:
             self.ops.rope_inplace(k, positions, self.cos, self.sin)
+
+
+@register(POSITIONS, "rope_interleaved")
+class InterleavedRotation(PositionEncoding):
+    """Rotation of the pairs (2i, 2i+1) of a vector's first `dims` dimensions by the angle
+    position * base^(-2i/dims); the rest passes unchanged.  The pair (u, v) becomes
+    (u cos a - v sin a, v cos a + u sin a).  There is no table and so no longest position:
+    kernels take `frequencies()` (float32 [dims/2], rounded once from float64) and compute
+    the angle and its cosine and sine in float32 at the position they need.
+
+    params: dims, base."""
+
+    def __init__(self, params, ctx):
+        super().__init__(params, ctx)
+        self.dims = int(params["dims"])
+        self.base = float(params["base"])
+        if self.dims % 2 or self.dims < 2:
+            raise ValueError(f"rotated dimensions must be even and at least 2, got {self.dims}")
+        i = torch.arange(self.dims // 2, dtype=torch.float64)
+        self.freqs = (self.base ** (-2.0 * i / self.dims)).to(torch.float32).to(ctx.device)
+
+    def frequencies(self):
+        return self.freqs
+
+    def step_read_tensors(self):
+        return []
+
+    def apply(self, q, k, positions):
+        self.ops.rotate_interleaved_inplace(q, positions, self.freqs, self.dims)
+        if k is not None:
+            self.ops.rotate_interleaved_inplace(k, positions, self.freqs, self.dims)

@@ -46,7 +46,10 @@ def random_tensors(raw_config: dict, seed: int, dtype=torch.float32, std: float 
         if decl.optional:
             continue
         gen = torch.Generator(device=device).manual_seed(_tensor_seed(seed, name))
-        if decl.role == "vector":
+        if decl.init is not None:
+            lo, hi = decl.init
+            t = lo + torch.rand(decl.shape, generator=gen, device=device) * (hi - lo)
+        elif decl.role == "vector":
             t = 1.0 + (torch.rand(decl.shape, generator=gen, device=device) * 0.2 - 0.1)
         elif decl.role == "table":
             raise ValueError(f"no random rule for integer table {name}")
