@@ -89,7 +89,7 @@ def main(args) -> None:
         _, model = random_model(raw, 0, args.dtype, "cuda:0")
         model_dir = tempfile.gettempdir()
     spec = model.spec
-    max_model_len = args.max_model_len or int(spec.max_position)
+    max_model_len = args.max_model_len or min(int(spec.max_position), 40960)
     if max_model_len > spec.max_position:
         raise ValueError(f"max_model_len cannot exceed the model's {spec.max_position}")
     limit = min(args.max_prompt_token_id, spec.vocab_size - 1)

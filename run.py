@@ -105,7 +105,9 @@ def main(args) -> None:
         eos = spec.eos_token_id if spec.eos_token_id is not None else -1
 
     config = Config(
-        model=str(model_dir), max_model_len=args.max_model_len or int(spec.max_position),
+        model=str(model_dir),
+        # a model without a longest position (no table to run out of) gets the engine's default
+        max_model_len=args.max_model_len or min(int(spec.max_position), 40960),
         eos=eos, dtype=dtype, enforce_eager=args.enforce_eager,
         kvcache_block_size=args.page_size, num_kvcache_blocks=args.num_pages,
         max_num_batched_tokens=args.max_num_batched_tokens, max_num_seqs=args.max_num_seqs,

@@ -90,3 +90,78 @@ def write_word_tokenizer(model_dir, vocab_size, *, eos_id=2, name_eos=True, pad_
         named["pad_token"] = "<pad>"
     (model_dir / "tokenizer_config.json").write_text(json.dumps(named))
     return tok
+
+
+# ------------------------------------------------------------------ Zonopel
+
+
+def zonopel_mamba(*, heads, vdim, state, groups, conv, norm_groups, ff=None, weights_of=None):
+    entry = {"type": "mamba2",
+             "mixer": {"heads": heads, "vdim": vdim, "state": state, "groups": groups,
+                       "conv": conv, "norm_groups": norm_groups},
+             "mlp": None if ff is None else {"kind": "dense", "ff": ff}}
+    if weights_of is not None:
+        entry["weights_of"] = weights_of
+    return entry
+
+
+def zonopel_latent(*, heads, dim, rot_dim, vdim, q_rank, kv_rank, window, base=10000.0,
+                   rot_dims=None, scale=None, ff=None, weights_of=None):
+    mixer = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "q_rank": q_rank,
+             "kv_rank": kv_rank, "scale": scale or (dim + rot_dim) ** -0.5,
+             "rot": {"base": base, "dims": rot_dims or rot_dim}}
+    if window is not None:
+        mixer["mask"] = {"size": window}
+    entry = {"type": "latent_attention", "mixer": mixer,
+             "mlp": None if ff is None else {"kind": "dense", "ff": ff}}
+    if weights_of is not None:
+        entry["weights_of"] = weights_of
+    return entry
+
+
+def zonopel_config(*, width, vocab, eps, scale, buckets, mul_prev, mul_cur, layers):
+    import copy
+    layers = copy.deepcopy(layers)
+    for entry in layers:            # a layer that borrows weights repeats the lender's entry
+        if "weights_of" in entry:
+            src = layers[entry["weights_of"]]
+            entry.update(type=src["type"], mixer=copy.deepcopy(src["mixer"]),
+                         mlp=copy.deepcopy(src["mlp"]))
+    return {"architecture": "Zonopel", "width": width, "vocab": vocab, "norm": {"eps": eps},
+            "embedding": {"scale": scale, "bigram": {"buckets": buckets, "mul_prev": mul_prev,
+                                                     "mul_cur": mul_cur}},
+            "layers": layers}
+
+
+# Three small models that differ in every size and option: windows of 5 tokens, of 17 and
+# none, a window of one token, partial rotation, heads that are no multiple of four, groups
+# equal to heads and one group, one and several norm groups, convolutions of 1, 2 and 4
+# taps, vdim above and below a workgroup's 32 columns, layers without a feed-forward,
+# borrowed weights in both mixers, an embedding scale of 1.
+ZONO_A = zonopel_config(
+    width=40, vocab=97, eps=1e-5, scale=2.5, buckets=61, mul_prev=31, mul_cur=5, layers=[
+        zonopel_latent(heads=3, dim=8, rot_dim=6, rot_dims=4, vdim=10, q_rank=12, kv_rank=14,
+                       window=5, ff=56),
+        zonopel_mamba(heads=4, vdim=6, state=5, groups=4, conv=4, norm_groups=1, ff=48),
+        zonopel_mamba(heads=0, vdim=0, state=0, groups=0, conv=0, norm_groups=0, weights_of=1),
+        zonopel_latent(heads=0, dim=0, rot_dim=2, vdim=0, q_rank=0, kv_rank=0, window=None,
+                       weights_of=0),
+        zonopel_mamba(heads=2, vdim=12, state=9, groups=1, conv=3, norm_groups=2, ff=None),
+    ])
+ZONO_B = zonopel_config(
+    width=72, vocab=131, eps=3e-6, scale=1.0, buckets=200, mul_prev=7, mul_cur=1009, layers=[
+        zonopel_mamba(heads=2, vdim=40, state=20, groups=1, conv=2, norm_groups=4, ff=100),
+        zonopel_latent(heads=5, dim=16, rot_dim=8, vdim=12, q_rank=24, kv_rank=32, window=None,
+                       base=500.0, ff=90),
+        zonopel_latent(heads=2, dim=12, rot_dim=4, vdim=20, q_rank=16, kv_rank=24, window=17,
+                       scale=0.3, ff=None),
+        zonopel_mamba(heads=0, vdim=0, state=0, groups=0, conv=0, norm_groups=0, weights_of=0),
+    ])
+ZONO_C = zonopel_config(
+    width=32, vocab=64, eps=1e-4, scale=0.5, buckets=17, mul_prev=3, mul_cur=3, layers=[
+        zonopel_mamba(heads=1, vdim=16, state=8, groups=1, conv=1, norm_groups=1, ff=40),
+        zonopel_latent(heads=4, dim=4, rot_dim=2, vdim=4, q_rank=8, kv_rank=8, window=1, ff=40),
+        zonopel_latent(heads=1, dim=8, rot_dim=8, vdim=8, q_rank=8, kv_rank=16, window=33,
+                       ff=24),
+    ])
+ZONO = {"A": (ZONO_A, 11, 4), "B": (ZONO_B, 12, 16), "C": (ZONO_C, 13, 8)}   # cfg, seed, page

@@ -51,6 +51,20 @@ def page_bytes(groups: list[GroupLayout], page_size: int, dtype: torch.dtype) ->
                * g.head_dim * item for g in groups)
 
 
+def state_bytes(needs, num_slots: int) -> int:
+    """Bytes the fixed-size per-request states of all runs take for `num_slots` slots (and
+    the spare one)."""
+    total = 0
+    for need in needs:
+        for n in flat_needs(need):
+            if isinstance(n, SlotStateNeed):
+                count = 1
+                for d in n.shape:
+                    count *= d
+                total += (num_slots + 1) * count * torch.empty((), dtype=n.dtype).element_size()
+    return total
+
+
 @dataclass
 class LayerCache:
     """The cache of one run, as a mixer sees it."""

@@ -93,7 +93,7 @@ class ZonopelConfig:
     bigram_mul_cur: int
     layers: tuple[ZonopelLayer, ...]
     eos_token_id: int | None = None
-    max_position: int = 1 << 22
+    max_position: int = 1 << 20
     architecture: str = ARCHITECTURE
     raw: dict = field(default_factory=dict, compare=False, repr=False)
 
@@ -141,7 +141,9 @@ class ZonopelConfig:
                     raise ConfigError(f"config.json: layers[{i}] borrows the weights of layers"
                                       f"[{layer.weights_of}] but differs from it")
         eos = raw.get("eos_token_id")
-        max_pos = raw.get("max_position", 1 << 22)
+        # positions have no table to run out of; the bound keeps float32 angles exact in the
+        # position and is what an engine is told when nobody gives it a length
+        max_pos = raw.get("max_position", 1 << 20)
         return cls(width=width, vocab_size=vocab, eps=eps,
                    embed_scale=float(_need(emb, "scale", "embedding")),
                    bigram_buckets=_pos_int(bigram, "buckets", "embedding.bigram"),

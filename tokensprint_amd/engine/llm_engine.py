@@ -145,7 +145,11 @@ class LLMEngine:
             raise ValueError("num_kvcache_blocks must be given when there is no GPU to size from")
         steps = LLMEngine.measure_step_memory(model, config, graph_len)
         free, _ = torch.cuda.mem_get_info(device)
-        available = free * config.gpu_memory_utilization - steps
+        # fixed-size state per request (recurrent state, shifts): one row a slot and one
+        # spare, allocated beside the pages
+        from tokensprint_amd.cache.storage import state_bytes
+        states = state_bytes(model.cache_needs(), config.max_num_seqs)
+        available = free * config.gpu_memory_utilization - steps - states
         pages = ModelRunner.pages_that_fit(model, config.kvcache_block_size, int(available),
                                            config.dtype)
         # no request can use more than max_model_len tokens
