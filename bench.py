@@ -277,6 +277,155 @@ def prefill_flops(cfg, layers, T) -> float:
     return layers * (per_token * T + prefill_attention_flops(cfg, T)) + 2 * H * V   # head: last token only
 
 
+# ------------------------------------------------------------------ Zonopel beside Qwen3
+# Sizes that resemble the layers of real models, the same width, depth, feed-forward size
+# and vocabulary for both designs.  Zonopel layers alternate (three Mamba-2, one latent
+# attention with a window), as hybrids of the two are built.
+COMPARE_SIZES = {
+    "1b-layers": dict(width=2048, layers=8, ff=8192, vocab=32000, heads=16, head_dim=128,
+                      kv_heads=8, ssm_heads=64, ssm_vdim=64, ssm_state=128, ssm_groups=8,
+                      q_rank=768, kv_rank=512, rot_dim=64, window=1024),
+    "0.5b-layers": dict(width=1024, layers=8, ff=4096, vocab=32000, heads=16, head_dim=64,
+                        kv_heads=8, ssm_heads=32, ssm_vdim=64, ssm_state=64, ssm_groups=4,
+                        q_rank=384, kv_rank=256, rot_dim=32, window=512),
+}
+
+
+def compare_configs(s):
+    mamba = {"type": "mamba2", "mlp": {"kind": "dense", "ff": s["ff"]},
+             "mixer": {"heads": s["ssm_heads"], "vdim": s["ssm_vdim"], "state": s["ssm_state"],
+                       "groups": s["ssm_groups"], "conv": 4, "norm_groups": s["ssm_groups"]}}
+    latent = {"type": "latent_attention", "mlp": {"kind": "dense", "ff": s["ff"]},
+              "mixer": {"heads": s["heads"], "dim": s["head_dim"], "rot_dim": s["rot_dim"],
+                        "vdim": s["head_dim"], "q_rank": s["q_rank"], "kv_rank": s["kv_rank"],
+                        "scale": (s["head_dim"] + s["rot_dim"]) ** -0.5,
+                        "rot": {"base": 10000.0, "dims": s["rot_dim"]},
+                        "mask": {"size": s["window"]}}}
+    zono = {"architecture": "Zonopel", "width": s["width"], "vocab": s["vocab"],
+            "norm": {"eps": 1e-5},
+            "embedding": {"scale": 1.0, "bigram": {"buckets": 16381, "mul_prev": 31337,
+                                                   "mul_cur": 7}},
+            "layers": [dict(latent if i % 4 == 3 else mamba) for i in range(s["layers"])]}
+    qwen = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+            "hidden_size": s["width"], "num_hidden_layers": s["layers"],
+            "num_attention_heads": s["heads"], "num_key_value_heads": s["kv_heads"],
+            "head_dim": s["head_dim"], "intermediate_size": 64,
+            "vocab_size": s["vocab"], "rms_norm_eps": 1e-6, "rope_theta": 1e6,
+            "max_position_embeddings": 8192, "tie_word_embeddings": False}
+    # equal size: the Qwen3 feed-forward takes up what its smaller mixer leaves
+    import math
+    from tokensprint_amd.weights.random_init import declared_tensors
+
+    def count(raw):
+        return sum(math.prod(d.shape) for d in declared_tensors(raw).values())
+    spare = count(zono) - count(qwen)
+    qwen["intermediate_size"] = 64 + max(0, round(spare / (3 * s["width"] * s["layers"]) / 64)) * 64
+    return zono, qwen
+
+
+class TimedOps:
+    """Wraps a kernel provider: every call of one of its operations is bracketed by events,
+    and `seconds` sums them per operation name (an eager step's kernels, one by one)."""
+
+    def __init__(self, ops):
+        import torch
+        self._ops, self._torch, self.pairs = ops, torch, []
+
+    def __getattr__(self, name):
+        attr = getattr(self._ops, name)
+        if not callable(attr) or name.startswith("_") or name in ("timed_plans", "reset_scratch"):
+            return attr
+
+        def timed(*a, **k):
+            start = self._torch.cuda.Event(enable_timing=True)
+            end = self._torch.cuda.Event(enable_timing=True)
+            start.record()
+            out = attr(*a, **k)
+            end.record()
+            self.pairs.append((name, start, end))
+            return out
+        return timed
+
+    def seconds(self):
+        self._torch.cuda.synchronize()
+        out = {}
+        for name, a, b in self.pairs:
+            out[name] = out.get(name, 0.0) + a.elapsed_time(b) * 1e-3
+        self.pairs = []
+        return out
+
+
+def op_times(model, page, entries_of, reps=3):
+    """Seconds per operation name of the eager step `entries_of` describes (the median run's)."""
+    from tokensprint_amd.engine.runner import ModelRunner
+    lengths = entries_of(None)
+    pages = sum(-(-n // page) + 1 for n in lengths)
+    runner = ModelRunner(model, page_size=page, num_pages=pages, num_slots=len(lengths))
+    batch = runner.build(entries_of(runner))
+    real = model.ctx.ops
+    timed = TimedOps(real)
+    parts = model.parts()
+    runs = []
+    try:
+        for part in parts:
+            part.ops = timed
+        model.ctx.ops = timed
+        for _ in range(reps + 1):
+            batch.plans.clear()
+            runner.run(batch)
+            runs.append(timed.seconds())
+    finally:
+        for part in parts:
+            part.ops = real
+        model.ctx.ops = real
+    runs = sorted(runs[1:], key=lambda r: sum(r.values()))
+    return runs[len(runs) // 2]
+
+
+def zonopel_compare(args) -> int:
+    """Prefill and decode throughput of Zonopel beside Qwen3 at equal sizes, and the time of
+    every kind of kernel in a 2,048-token prompt and in a decode step of eight requests.
+    Prints one JSON line of its own."""
+    import torch
+    from tokensprint_amd.engine.assemble import random_model
+    page, T, b, ctx = 16, 2048, 8, 2048
+    out = {"metric": "zonopel beside qwen3 at equal sizes (random weights, bf16)", "sizes": {}}
+    for name, size in COMPARE_SIZES.items():
+        if args.compare_size and name != args.compare_size:
+            continue
+        row = {}
+        for design, raw in zip(("zonopel", "qwen3"), compare_configs(size)):
+            _, model = random_model(raw, 0, args.dtype, "cuda:0")
+            vocab = size["vocab"]
+            _, engine = make_engine(raw, args.dtype, None, 1, 4096, T, page, model=model)
+            pre = prefill_run(engine, T, vocab)
+            del engine
+            steps, warmup = 64, 8
+            max_len, max_tokens = decode_lengths(b, ctx - 128, steps, warmup, 4096)
+            _, engine = make_engine(raw, args.dtype, None, b, max_len, 4096, page, model=model)
+            sec, decoded, held = decode_run(engine, b, ctx - 128, steps, warmup, vocab, max_tokens)
+            del engine
+            params = sum(t.numel() for part in model.parts() for t in part.held_tensors()
+                         if t.dim() == 2)
+            row[design] = {
+                "matrix_params_m": round(params / 1e6, 1),
+                "prefill_tok_s": round(T / pre, 1), "prefill_ms": round(pre * 1e3, 3),
+                "decode_tok_s": round(decoded / sec, 1),
+                "decode_ms_step": round(sec / steps * 1e3, 4),
+                "decode_frac_hbm": round(model.step_weight_bytes() * steps / sec / 1e9
+                                         / HBM_PEAK_GBS, 4),
+                "prefill_op_us": {k: round(v * 1e6, 1) for k, v in sorted(
+                    op_times(model, page, prefill_entries(T)).items())},
+                "decode_op_us": {k: round(v * 1e6, 1) for k, v in sorted(
+                    op_times(model, page, decode_entries(b, ctx)).items())},
+            }
+            del model
+            torch.cuda.empty_cache()
+        out["sizes"][name] = row
+    print(json.dumps(out))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -294,6 +443,10 @@ def main() -> int:
     ap.add_argument("--skip-fp32", action="store_true", help="no float32 decode point")
     ap.add_argument("--only-prefill", action="store_true",
                     help="only the 2,048-token prefill (for profiling); prints its own line")
+    ap.add_argument("--compare-zonopel", action="store_true",
+                    help="instead of the benchmark: Zonopel beside Qwen3 at equal sizes "
+                         "(prefill, decode, time per kind of kernel); prints its own line")
+    ap.add_argument("--compare-size", default=None, help="with --compare-zonopel: one size only")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -302,6 +455,8 @@ def main() -> int:
     import torch
     from tokensprint_amd.config import load_named_config
 
+    if args.compare_zonopel:
+        return zonopel_compare(args)
     raw = load_named_config(args.model)
     full_layers = raw["num_hidden_layers"]
     layers = args.layers or full_layers

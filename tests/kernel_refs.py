@@ -253,8 +253,9 @@ class TorchOps:
         out[..., 1:dims:2] = b * cos + a * sin
         return out
 
-    def rotate_interleaved_inplace(self, x, positions, freqs, dims):
-        x.copy_(self._rotate_pairs(x.float(), positions, freqs, dims).to(x.dtype))
+    def rotate_interleaved_inplace(self, x, positions, freqs, dims, offset=0):
+        part = x[..., offset:]
+        part.copy_(self._rotate_pairs(part.float(), positions, freqs, dims).to(x.dtype))
 
     def latent_prepare(self, proj, batch, table, cache, *, q_rank, kv_rank, rot_dim, q_norm,
                        kv_norm, eps, freqs, rot_dims, out_dtype):
@@ -270,16 +271,8 @@ class TorchOps:
         cache.k_pages[page, pos % P] = torch.cat([c, kr], dim=-1).to(cache.k_pages.dtype)
         return cq.to(out_dtype)
 
-    def latent_query(self, q, w_uk, batch, *, heads, dim, rot_dim, kv_rank, freqs, rot_dims):
-        T = q.shape[0]
-        q = q.float().view(T, heads, dim + rot_dim)
-        uk = w_uk.float().view(heads, dim, kv_rank)
-        ql = torch.einsum("thd,hdr->thr", q[..., :dim], uk)
-        qr = self._rotate_pairs(q[..., dim:], batch.positions, freqs, rot_dims)
-        return torch.cat([ql, qr], dim=-1).contiguous()
-
     def latent_attention(self, qa, batch, table, cache, *, heads, kv_rank, rot_dim, scale,
-                         window):
+                         window, out_dtype=torch.float32):
         T = qa.shape[0]
         P = cache.page_size
         out = torch.empty(T, heads, kv_rank, dtype=torch.float32, device=qa.device)
@@ -293,12 +286,7 @@ class TorchOps:
             kv = cache.k_pages[pages, keys % P].float()          # [n, kv_rank + rot_dim]
             s = (kv @ qa[t].float().T) * scale                   # [n, heads]
             out[t] = torch.softmax(s, dim=0).T @ kv[:, :kv_rank]
-        return out
-
-    def head_linear(self, x, weight, heads, out_dtype):
-        T = x.shape[0]
-        w = weight.float().view(heads, -1, x.shape[-1])          # [heads, out, in]
-        return torch.einsum("thr,hor->tho", x.float(), w).reshape(T, -1).to(out_dtype)
+        return out.to(out_dtype)
 
     # ---------------------------------------------------------------- sampling
     def argmax(self, logits):

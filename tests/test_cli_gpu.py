@@ -123,3 +123,23 @@ def test_model_registry_py():
     assert "qwen:\n  - qwen3-0.6b (qwen/qwen3-0.6b)" in proc.stdout
     assert "tiny" not in proc.stdout               # test configurations are no presets
     assert "Qwen3ForCausalLM" in proc.stdout
+
+
+def test_run_py_serves_a_zonopel_model(gpu_device, tmp_path):
+    """config.json names the architecture; run.py, the engine (pages sized from free
+    memory, state slots, captured decode steps) and the sampler serve it as any other."""
+    from helpers import ZONO_B
+    from plain import zonopel_plain
+    prompt = random_prompt(21, ZONO_B["vocab"], 9)
+    model_dir = tmp_path / "zono-b"
+    proc = run_program(["run.py", "--config-json", config_json(tmp_path, ZONO_B),
+                        "--random-weights", "2", "--model-dir", model_dir, "--dtype", "float32",
+                        "--temperature", "0", "--max-tokens", "9", "--ignore-eos", "True",
+                        "--max-num-seqs", "8", "--max-model-len", "256",
+                        "--prompt-ids", ",".join(map(str, prompt))])
+    got = json.loads(proc.stdout.strip().splitlines()[-1])
+    pcfg, w = zonopel_plain.read_model_dir(model_dir)
+    tokens = list(prompt)
+    for _ in range(9):
+        tokens.append(int(zonopel_plain.forward(pcfg, w, tokens)[-1].argmax()))
+    assert got == tokens[len(prompt):]

@@ -164,6 +164,31 @@ def test_convolution_and_recurrence_over_steps(gpu_device, heads, vdim, N, group
                   REF.gated_group_norm(y_ref, proj, nw, g, 1e-5, torch.float32))
 
 
+def test_long_portions_run_in_chunks(gpu_device):
+    """Portions above the chunking threshold (cut into runs of 64 tokens side by side)
+    beside short ones, continued over steps: the same y and state as the plain walk."""
+    ops = load_hip_ops(gpu_device)
+    heads, vdim, N, groups = 3, 40, 20, 1
+    inner = heads * vdim
+    scene = Scene(gpu_device, SlotStateNeed((heads, N, vdim), torch.float32, "ssm"), 16, 4,
+                  num_pages=80)
+    state = scene.view.states["ssm"]
+    state.fill_(5.0)
+    ref_state = state.clone()
+    dt_bias, a_log = rnd((heads,), 3).to(gpu_device) - 2, rnd((heads,), 4, 0.5).to(gpu_device) - 1
+    d_skip = rnd((heads,), 5).to(gpu_device)
+    for i, spans in enumerate([[300, 1, 130, 64], [1, 200, 2, 129], [129, 0, 1, 1]]):
+        batch = scene.step(spans)
+        assert batch.max_q_len > ops.dispatch.scan_whole_tokens
+        xbc = rnd((batch.num_tokens, inner + 2 * groups * N), 50 + i, 0.5).to(gpu_device)
+        proj = rnd((batch.num_tokens, heads), 60 + i).to(gpu_device)
+        kw = dict(heads=heads, vdim=vdim, state_rows=N, groups=groups)
+        y = ops.ssm_scan(xbc, proj, 0, dt_bias, a_log, d_skip, batch, state, **kw)
+        y_ref = REF.ssm_scan(xbc, proj, 0, dt_bias, a_log, d_skip, batch, ref_state, **kw)
+        close(y, y_ref, rtol=1e-4, atol=1e-4)
+        close(state, ref_state, rtol=1e-4, atol=1e-4)
+
+
 def test_recurrence_remembers_a_far_token(gpu_device):
     """With a decay of almost one, what one early token wrote is read hundreds of tokens
     later, across steps; with a strong decay it is gone."""
@@ -207,8 +232,6 @@ def test_latent_attention_kernels(gpu_device, cache_dtype, heads, dim, rot_dim, 
     ref_view = dataclasses.replace(scene.view, k_pages=ref_pages)
     freqs = (10000.0 ** (-2.0 * torch.arange(rot_dims // 2) / rot_dims)).float().to(gpu_device)
     qn, kn = (1 + 0.1 * rnd((q_rank,), 1)).to(gpu_device), (1 + 0.1 * rnd((kv_rank,), 2)).to(gpu_device)
-    uk = rnd((heads * dim, kv_rank), 3, 0.2).to(cache_dtype).to(gpu_device)
-    uv = rnd((heads * vdim, kv_rank), 4, 0.2).to(cache_dtype).to(gpu_device)
     tol = dict(rtol=1e-4, atol=1e-4) if cache_dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
     for i, spans in enumerate(SPANS):
         batch = scene.step(spans)
@@ -221,16 +244,17 @@ def test_latent_attention_kernels(gpu_device, cache_dtype, heads, dim, rot_dim, 
               REF.latent_prepare(proj, batch, table, ref_view, **kw))
         close(scene.view.k_pages, ref_pages, **tol)
         ref_pages.copy_(scene.view.k_pages)       # attention below reads identical pages
-        q = rnd((T, heads * (dim + rot_dim)), 40 + i).to(gpu_device)
-        kw = dict(heads=heads, dim=dim, rot_dim=rot_dim, kv_rank=kv_rank, freqs=freqs,
-                  rot_dims=rot_dims)
-        qa = REF.latent_query(q, uk, batch, **kw)
-        close(ops.latent_query(q, uk, batch, **kw), qa, rtol=1e-4, atol=1e-4)
+        qa = rnd((T, heads, dl), 40 + i).to(gpu_device)
+        qb = qa.clone()
+        ops.rotate_interleaved_inplace(qa, batch.positions, freqs, rot_dims, offset=kv_rank)
+        REF.rotate_interleaved_inplace(qb, batch.positions, freqs, rot_dims, offset=kv_rank)
+        close(qa, qb)
         kw = dict(heads=heads, kv_rank=kv_rank, rot_dim=rot_dim, scale=0.2, window=window)
-        ol = REF.latent_attention(qa, batch, table, ref_view, **kw)
-        close(ops.latent_attention(qa, batch, table, scene.view, **kw), ol, rtol=1e-4, atol=1e-4)
-        close(ops.head_linear(ol, uv, heads, torch.float32),
-              REF.head_linear(ol, uv, heads, torch.float32), rtol=1e-4, atol=1e-4)
+        ol = REF.latent_attention(qb, batch, table, ref_view, **kw)
+        close(ops.latent_attention(qb, batch, table, scene.view, **kw), ol, **tol)
+        got = ops.latent_attention(qb, batch, table, scene.view, out_dtype=torch.bfloat16, **kw)
+        assert got.dtype == torch.bfloat16
+        close(got, ol, rtol=2e-2, atol=2e-2)
 
 
 @pytest.mark.parametrize("window", [None, 20, 64, 65])

@@ -4,8 +4,9 @@
 // result leaves as sum_t p_t c_t per head, for the value up-projection behind it.
 //
 // Kernels: the preparation of a step's rows (norms of the two latents, rotation of the
-// shared key part, the write into the pages), the carrying of queries into the latent's
-// space, attention, and the per-head product that carries results back out.
+// shared key part, the write into the pages), the rotation of the queries' rotated part in
+// place, and attention.  (Carrying queries into the latent's space and results out of it
+// are plain products over weights folded at load.)
 // Scores, softmax, rotation angles, norms: float32.  The rotation pairs dimension 2i with
 // 2i+1 and turns them by position * freq[i]; cosine and sine are computed here, at the
 // position, so there is no table and no longest position.
@@ -89,69 +90,38 @@ extern "C" int ts_latent_prepare(const float* proj, const float* q_norm, const f
   return 0;
 }
 
-// ---------------------------------------------------------------- queries into the latent's space
-// q [T, heads, dim + rot_dim] float32; U_k [heads * dim, kv_rank].
-// out[t, h] = [ sum_d q[t, h, d] U_k[h * dim + d, :]  |  rot(q[t, h, dim:]) ], float32.
-// A workgroup serves one head and eight tokens, so a row of U_k is read once for eight.
-constexpr int kQueryTile = 8;
-
-template <typename TW>
-__global__ __launch_bounds__(256) void latent_query_kernel(
-    const float* __restrict__ q, const TW* __restrict__ uk, const float* __restrict__ freqs,
-    const int* __restrict__ positions, float* __restrict__ out, int num_tokens, int heads,
-    int dim, int rot_dim, int kv_rank, int rot_dims) {
-  extern __shared__ float q_s[];     // [kQueryTile][dim]
-  const int h = blockIdx.x, t0 = blockIdx.y * kQueryTile;
-  const int qd = dim + rot_dim, dl = kv_rank + rot_dim;
-  const int nt = min(kQueryTile, num_tokens - t0);
-  for (int i = threadIdx.x; i < kQueryTile * dim; i += blockDim.x) {
-    const int tt = i / dim, d = i % dim;
-    q_s[i] = tt < nt ? q[((int64_t)(t0 + tt) * heads + h) * qd + d] : 0.f;
-  }
-  __syncthreads();
-  const TW* w = uk + (int64_t)h * dim * kv_rank;
-  for (int r = threadIdx.x; r < kv_rank; r += blockDim.x) {
-    float acc[kQueryTile] = {};
-    for (int d = 0; d < dim; ++d) {
-      const float wv = to_f32(w[(int64_t)d * kv_rank + r]);
-#pragma unroll
-      for (int tt = 0; tt < kQueryTile; ++tt) acc[tt] = fmaf(q_s[tt * dim + d], wv, acc[tt]);
-    }
-#pragma unroll
-    for (int tt = 0; tt < kQueryTile; ++tt)
-      if (tt < nt) out[((int64_t)(t0 + tt) * heads + h) * dl + r] = acc[tt];
-  }
-  const int pairs = rot_dim / 2 + rot_dim % 2;
-  for (int i = threadIdx.x; i < nt * pairs; i += blockDim.x) {
-    const int tt = i / pairs, j = i % pairs;
-    const float* src = q + ((int64_t)(t0 + tt) * heads + h) * qd + dim;
-    float* dst = out + ((int64_t)(t0 + tt) * heads + h) * dl + kv_rank;
-    if (2 * j + 1 < rot_dims) {
-      rotate_pair(src[2 * j], src[2 * j + 1], positions[t0 + tt], freqs[j], &dst[2 * j],
-                  &dst[2 * j + 1]);
-    } else {
-      dst[2 * j] = src[2 * j];
-      if (2 * j + 1 < rot_dim) dst[2 * j + 1] = src[2 * j + 1];
-    }
-  }
+// ---------------------------------------------------------------- rotation in place
+// x [T, heads, width]: the pairs (offset + 2i, offset + 2i + 1), i < dims / 2, of every
+// head's vector are turned by positions[t] * freqs[i].
+template <typename T>
+__global__ __launch_bounds__(256) void rotate_interleaved_kernel(
+    T* __restrict__ x, const int* __restrict__ positions, const float* __restrict__ freqs,
+    int64_t total, int heads, int width, int offset, int half) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int i = (int)(idx % half);
+  const int64_t th = idx / half;                      // token * heads + head
+  T* v = x + th * width + offset + 2 * i;
+  float a, b;
+  rotate_pair(to_f32(v[0]), to_f32(v[1]), positions[th / heads], freqs[i], &a, &b);
+  v[0] = from_f32<T>(a);
+  v[1] = from_f32<T>(b);
 }
 
-extern "C" int ts_latent_query(const float* q, const void* uk, int weight_type,
-                               const float* freqs, const int* positions, float* out,
-                               int num_tokens, int heads, int dim, int rot_dim, int kv_rank,
-                               int rot_dims, hipStream_t stream) {
-  if (num_tokens <= 0) return 0;
-  if (heads <= 0 || dim <= 0 || kv_rank <= 0 || rot_dim < 0 || rot_dims % 2 || rot_dims > rot_dim)
-    TS_FAIL("latent_query: bad sizes heads=%d dim=%d rot_dim=%d kv_rank=%d", heads, dim, rot_dim,
-            kv_rank);
-  const size_t lds = (size_t)kQueryTile * dim * sizeof(float);
-  if (lds > 64 * 1024) TS_FAIL("latent_query: head size %d too large", dim);
-  const dim3 grid(heads, (num_tokens + kQueryTile - 1) / kQueryTile);
-  TS_DISPATCH_TYPE(weight_type, TW,
-                   hipLaunchKernelGGL(latent_query_kernel<TW>, grid, dim3(256), lds, stream, q,
-                                      (const TW*)uk, freqs, positions, out, num_tokens, heads, dim,
-                                      rot_dim, kv_rank, rot_dims));
-  TS_CHECK_LAUNCH("latent_query");
+extern "C" int ts_rotate_interleaved(void* x, int type, const int* positions, const float* freqs,
+                                     int num_tokens, int heads, int width, int offset, int dims,
+                                     hipStream_t stream) {
+  if (num_tokens <= 0 || dims == 0) return 0;
+  if (heads <= 0 || dims % 2 || offset < 0 || offset + dims > width)
+    TS_FAIL("rotate_interleaved: bad sizes heads=%d width=%d offset=%d dims=%d", heads, width,
+            offset, dims);
+  const int64_t total = (int64_t)num_tokens * heads * (dims / 2);
+  TS_DISPATCH_TYPE(type, T,
+                   hipLaunchKernelGGL(rotate_interleaved_kernel<T>,
+                                      dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                                      (T*)x, positions, freqs, total, heads, width, offset,
+                                      dims / 2));
+  TS_CHECK_LAUNCH("rotate_interleaved");
   return 0;
 }
 
@@ -165,9 +135,9 @@ constexpr int kMaxLatent = 1024;              // kv_rank + rot_dim
 constexpr int kLatentWaves = 4;
 constexpr int kMaxRankPerLane = 8;            // kv_rank <= 512
 
-template <typename TC>
+template <typename TC, typename TO>
 __global__ __launch_bounds__(kLatentWaves* kWave) void latent_attention_kernel(
-    const float* __restrict__ qa, const TC* __restrict__ pages, float* __restrict__ out,
+    const float* __restrict__ qa, const TC* __restrict__ pages, TO* __restrict__ out,
     const int* __restrict__ positions, const int* __restrict__ entry_of_token,
     const int* __restrict__ table, int table_width, int page_size, int heads, int kv_rank,
     int rot_dim, int window, float scale) {
@@ -236,17 +206,17 @@ __global__ __launch_bounds__(kLatentWaves* kWave) void latent_attention_kernel(
     }
     __builtin_amdgcn_wave_barrier();
   }
-  float* o = out + ((int64_t)t * heads + h) * kv_rank;
+  TO* o = out + ((int64_t)t * heads + h) * kv_rank;
   const float inv = l > 0.f ? 1.0f / l : 0.f;
 #pragma unroll
   for (int r = 0; r < kMaxRankPerLane; ++r) {
     const int d = lane + r * kWave;
-    if (d < kv_rank) o[d] = acc[r] * inv;
+    if (d < kv_rank) o[d] = from_f32<TO>(acc[r] * inv);
   }
 }
 
-extern "C" int ts_latent_attention(const float* qa, const void* pages, int cache_type, float* out,
-                                   const int* positions, const int* entry_of_token,
+extern "C" int ts_latent_attention(const float* qa, const void* pages, int cache_type, void* out,
+                                   int out_type, const int* positions, const int* entry_of_token,
                                    const int* table, int table_width, int page_size,
                                    int num_tokens, int heads, int kv_rank, int rot_dim,
                                    int window, float scale, hipStream_t stream) {
@@ -259,59 +229,11 @@ extern "C" int ts_latent_attention(const float* qa, const void* pages, int cache
             rot_dim, kMaxRankPerLane * kWave, kMaxLatent - kMaxRankPerLane * kWave);
   const size_t lds = (size_t)kLatentWaves * (dl + 2 * kWave) * sizeof(float);
   const dim3 grid(num_tokens, (heads + kLatentWaves - 1) / kLatentWaves);
-  TS_DISPATCH_TYPE(cache_type, TC,
-                   hipLaunchKernelGGL(latent_attention_kernel<TC>, grid,
-                                      dim3(kLatentWaves * kWave), lds, stream, qa, (const TC*)pages,
-                                      out, positions, entry_of_token, table, table_width,
-                                      page_size, heads, kv_rank, rot_dim, window, scale));
+  TS_DISPATCH_TYPE(cache_type, TC, TS_DISPATCH_TYPE(out_type, TO,
+      hipLaunchKernelGGL((latent_attention_kernel<TC, TO>), grid, dim3(kLatentWaves * kWave), lds,
+                         stream, qa, (const TC*)pages, (TO*)out, positions, entry_of_token, table,
+                         table_width, page_size, heads, kv_rank, rot_dim, window, scale)));
   TS_CHECK_LAUNCH("latent_attention");
   return 0;
 }
 
-// ---------------------------------------------------------------- per-head product
-// x [T, heads, in] float32; W [heads * rows, in]; out[t, h, j] = sum_r W[h * rows + j, r]
-// x[t, h, r].  A workgroup serves one head and eight tokens; a wavefront takes a row of W,
-// its lanes stride over r, and the eight sums are added through the wavefront.
-template <typename TW, typename TO>
-__global__ __launch_bounds__(256) void head_linear_kernel(
-    const float* __restrict__ x, const TW* __restrict__ w, TO* __restrict__ out, int num_tokens,
-    int heads, int rows, int in) {
-  extern __shared__ float x_s[];      // [kQueryTile][in]
-  const int h = blockIdx.x, t0 = blockIdx.y * kQueryTile;
-  const int nt = min(kQueryTile, num_tokens - t0);
-  for (int i = threadIdx.x; i < kQueryTile * in; i += blockDim.x) {
-    const int tt = i / in, r = i % in;
-    x_s[i] = tt < nt ? x[((int64_t)(t0 + tt) * heads + h) * in + r] : 0.f;
-  }
-  __syncthreads();
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  for (int j = wave; j < rows; j += blockDim.x / kWave) {
-    const TW* wr = w + ((int64_t)h * rows + j) * in;
-    float acc[kQueryTile] = {};
-    for (int r = lane; r < in; r += kWave) {
-      const float wv = to_f32(wr[r]);
-#pragma unroll
-      for (int tt = 0; tt < kQueryTile; ++tt) acc[tt] = fmaf(x_s[tt * in + r], wv, acc[tt]);
-    }
-#pragma unroll
-    for (int tt = 0; tt < kQueryTile; ++tt) {
-      const float v = wave_sum(acc[tt]);
-      if (lane == 0 && tt < nt) out[((int64_t)(t0 + tt) * heads + h) * rows + j] = from_f32<TO>(v);
-    }
-  }
-}
-
-extern "C" int ts_head_linear(const float* x, const void* w, int weight_type, void* out,
-                              int out_type, int num_tokens, int heads, int rows, int in,
-                              hipStream_t stream) {
-  if (num_tokens <= 0) return 0;
-  if (heads <= 0 || rows <= 0 || in <= 0) TS_FAIL("head_linear: bad sizes");
-  const size_t lds = (size_t)kQueryTile * in * sizeof(float);
-  if (lds > 64 * 1024) TS_FAIL("head_linear: rows of %d elements too long", in);
-  const dim3 grid(heads, (num_tokens + kQueryTile - 1) / kQueryTile);
-  TS_DISPATCH_TYPE(weight_type, TW, TS_DISPATCH_TYPE(out_type, TO,
-      hipLaunchKernelGGL((head_linear_kernel<TW, TO>), grid, dim3(256), lds, stream, x,
-                         (const TW*)w, (TO*)out, num_tokens, heads, rows, in)));
-  TS_CHECK_LAUNCH("head_linear");
-  return 0;
-}

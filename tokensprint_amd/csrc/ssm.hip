@@ -142,10 +142,17 @@ extern "C" int ts_conv_silu(const float* proj, int ld, int col, int channels, in
 // ---------------------------------------------------------------- recurrence
 // Per head h (group g): d = softplus(dt + dt_bias[h]), a = exp(-exp(A_log[h]) d),
 //   S <- a S + (d B_g) x_h^T   (S: N x P),   y_h = S^T C_g + D[h] x_h.
-// A workgroup serves one (entry, head, 32 columns of P): thread (p, s) keeps rows
-// s, s + 8, ... of column p in registers, walks the entry's tokens in order and adds the
-// eight slices of a column's dot product through the wavefront.  The operands of the next
-// token are fetched while the current one is computed.
+// A workgroup serves one (run of tokens, head, 32 columns of P): thread (p, s) keeps rows
+// s, s + 8, ... of column p in registers, walks the tokens in order and adds the eight
+// slices of a column's dot product through the wavefront.  The operands of the next token
+// are fetched while the current one is computed.
+//
+// Steps of few tokens per entry walk each entry whole (kScanWhole).  A long portion is cut
+// into chunks of 64 tokens that run side by side, in three launches: every chunk's
+// recurrence from an empty state (its own contribution and the product of its decays,
+// kScanLocal); per entry, the state in front of every chunk, one after the other, and the
+// state the portion leaves (combine); every chunk once more from its true start state,
+// now writing y (kScanOutput).  Twice the arithmetic, a sixty-fourth of the chain.
 struct ScanArgs {
   const float* xbc;       // [T, channels]: x (heads*P) | B (groups*N) | C (groups*N)
   const float* proj;      // [T, ld]: dt at column dt_col
@@ -156,25 +163,41 @@ struct ScanArgs {
   float* y;               // [T, heads*P]
   BatchView b;
   int ld, dt_col, channels, heads, P, N, groups;
+  const int* chunks;      // [num_chunks, 3]: first token, one past the last, entry
+  const int* entry_chunks;  // [B + 1]: the chunks of entry e are [entry_chunks[e], entry_chunks[e+1])
+  float* chunk_state;     // [num_chunks, heads, N, P]: local contribution, then start state
+  float* chunk_decay;     // [num_chunks, heads]
 };
 
 constexpr int kScanSlices = 8;
 constexpr int kScanCols = 32;
+constexpr int kScanWhole = 0, kScanLocal = 1, kScanOutput = 2;
 
-template <int NI>
+template <int NI, int MODE>
 __global__ __launch_bounds__(kScanSlices* kScanCols) void ssm_scan_kernel(ScanArgs a) {
-  const int h = blockIdx.x, e = blockIdx.y;
+  const int h = blockIdx.x;
   const int p = blockIdx.z * kScanCols + threadIdx.x / kScanSlices;
   const int s = threadIdx.x % kScanSlices;
   const bool live = p < a.P;
   const int pc = live ? p : a.P - 1;      // idle columns shadow the last one and store nothing
   const int g = h / (a.heads / a.groups);
-  const int first = a.b.q_start[e], end = a.b.q_start[e + 1];
+  int first, end, e;
+  if (MODE == kScanWhole) {
+    e = blockIdx.y;
+    first = a.b.q_start[e];
+    end = a.b.q_start[e + 1];
+  } else {
+    first = a.chunks[3 * blockIdx.y];
+    end = a.chunks[3 * blockIdx.y + 1];
+    e = a.chunks[3 * blockIdx.y + 2];
+  }
   const int inner = a.heads * a.P;
   const int N = a.N;
-  float* st = a.state + ((int64_t)a.b.slot_ids[e] * a.heads + h) * N * a.P;
+  float* st = MODE == kScanWhole
+      ? a.state + ((int64_t)a.b.slot_ids[e] * a.heads + h) * N * a.P
+      : a.chunk_state + ((int64_t)blockIdx.y * a.heads + h) * N * a.P;
   float S[NI];
-  const bool fresh = a.b.positions[first] == 0;
+  const bool fresh = MODE == kScanLocal || (MODE == kScanWhole && a.b.positions[first] == 0);
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
     const int n = s + kScanSlices * i;
@@ -193,19 +216,29 @@ __global__ __launch_bounds__(kScanSlices* kScanCols) void ssm_scan_kernel(ScanAr
     for (int i = 0; i < NI; ++i) {
       const int n = s + kScanSlices * i;
       nB[i] = n < N ? row[b_col + n] : 0.f;
-      nC[i] = n < N ? row[c_col + n] : 0.f;
+      if (MODE != kScanLocal) nC[i] = n < N ? row[c_col + n] : 0.f;
     }
   };
   if (first < end) fetch(first);
+  float total_decay = 1.f;
   for (int t = first; t < end; ++t) {
     float B[NI], C[NI];
     const float x = nx, dt_raw = ndt;
 #pragma unroll
-    for (int i = 0; i < NI; ++i) { B[i] = nB[i]; C[i] = nC[i]; }
+    for (int i = 0; i < NI; ++i) {
+      B[i] = nB[i];
+      if (MODE != kScanLocal) C[i] = nC[i];
+    }
     if (t + 1 < end) fetch(t + 1);
     const float d = softplus_f(dt_raw + bias);
     const float decay = expf(decay_rate * d);
     const float dx = d * x;
+    if (MODE == kScanLocal) {
+      total_decay *= decay;
+#pragma unroll
+      for (int i = 0; i < NI; ++i) S[i] = fmaf(decay, S[i], B[i] * dx);
+      continue;
+    }
     float acc = 0.f;
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
@@ -217,6 +250,7 @@ __global__ __launch_bounds__(kScanSlices* kScanCols) void ssm_scan_kernel(ScanAr
     acc += __shfl_xor(acc, 4, kWave);
     if (s == 0 && live) a.y[(int64_t)t * inner + h * a.P + p] = fmaf(skip, x, acc);
   }
+  if (MODE == kScanOutput) return;
   if (live) {
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
@@ -224,30 +258,94 @@ __global__ __launch_bounds__(kScanSlices* kScanCols) void ssm_scan_kernel(ScanAr
       if (n < N) st[(int64_t)n * a.P + p] = S[i];
     }
   }
+  if (MODE == kScanLocal && blockIdx.z == 0 && threadIdx.x == 0)
+    a.chunk_decay[(int64_t)blockIdx.y * a.heads + h] = total_decay;
 }
 
+// Per (head, entry, 32 columns): walks the entry's chunks in order.  chunk_state[c] holds
+// the chunk's own contribution and receives the state in front of the chunk; the state
+// behind the last chunk goes to the request's slot.
+template <int NI>
+__global__ __launch_bounds__(kScanSlices* kScanCols) void ssm_combine_kernel(ScanArgs a) {
+  const int h = blockIdx.x, e = blockIdx.y;
+  const int p = blockIdx.z * kScanCols + threadIdx.x / kScanSlices;
+  const int s = threadIdx.x % kScanSlices;
+  if (p >= a.P) return;
+  const int N = a.N;
+  float* st = a.state + ((int64_t)a.b.slot_ids[e] * a.heads + h) * N * a.P;
+  const bool fresh = a.b.positions[a.b.q_start[e]] == 0;
+  float S[NI];
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+    const int n = s + kScanSlices * i;
+    S[i] = (!fresh && n < N) ? st[(int64_t)n * a.P + p] : 0.f;
+  }
+  for (int c = a.entry_chunks[e]; c < a.entry_chunks[e + 1]; ++c) {
+    float* cs = a.chunk_state + ((int64_t)c * a.heads + h) * N * a.P;
+    const float decay = a.chunk_decay[(int64_t)c * a.heads + h];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int n = s + kScanSlices * i;
+      if (n < N) {
+        const float local = cs[(int64_t)n * a.P + p];
+        cs[(int64_t)n * a.P + p] = S[i];
+        S[i] = fmaf(decay, S[i], local);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+    const int n = s + kScanSlices * i;
+    if (n < N) st[(int64_t)n * a.P + p] = S[i];
+  }
+}
+
+template <int NI>
+static void launch_scan(const ScanArgs& a, int num_entries, int num_chunks, hipStream_t stream) {
+  const dim3 block(kScanSlices * kScanCols);
+  const unsigned z = (a.P + kScanCols - 1) / kScanCols;
+  if (num_chunks <= 0) {
+    hipLaunchKernelGGL((ssm_scan_kernel<NI, kScanWhole>), dim3(a.heads, num_entries, z), block, 0,
+                       stream, a);
+    return;
+  }
+  hipLaunchKernelGGL((ssm_scan_kernel<NI, kScanLocal>), dim3(a.heads, num_chunks, z), block, 0,
+                     stream, a);
+  hipLaunchKernelGGL(ssm_combine_kernel<NI>, dim3(a.heads, num_entries, z), block, 0, stream, a);
+  hipLaunchKernelGGL((ssm_scan_kernel<NI, kScanOutput>), dim3(a.heads, num_chunks, z), block, 0,
+                     stream, a);
+}
+
+extern "C" int ts_ssm_scan_chunk() { return 64; }
+
+// `num_chunks` 0: every entry is walked whole.  Else `chunks` [num_chunks, 3] cuts every
+// entry into runs of tokens (first, one past the last, entry), in order, `entry_chunks`
+// [B + 1] says which are whose, and chunk_state [num_chunks, heads, N, P], chunk_decay
+// [num_chunks, heads] are scratch.
 extern "C" int ts_ssm_scan(const float* xbc, const float* proj, int ld, int dt_col,
                            const float* dt_bias, const float* a_log, const float* d_skip,
                            float* state, float* y, const int* positions,
                            const int* entry_of_token, const int* q_start, const int* slot_ids,
                            int num_tokens, int num_entries, int heads, int P, int N, int groups,
-                           hipStream_t stream) {
+                           const int* chunks, const int* entry_chunks, int num_chunks,
+                           float* chunk_state, float* chunk_decay, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (heads <= 0 || P <= 0 || N <= 0 || groups <= 0 || heads % groups)
     TS_FAIL("ssm_scan: bad sizes heads=%d vdim=%d state=%d groups=%d", heads, P, N, groups);
   if (N > kScanSlices * 32) TS_FAIL("ssm_scan: state of %d rows, at most %d are built", N, kScanSlices * 32);
   if (dt_col < 0 || dt_col + heads > ld) TS_FAIL("ssm_scan: dt columns outside the projection");
+  if (num_chunks > 0 && (!chunks || !entry_chunks || !chunk_state || !chunk_decay))
+    TS_FAIL("ssm_scan: chunked without its lists and scratch");
   ScanArgs a{xbc, proj, dt_bias, a_log, d_skip, state, y,
              BatchView{positions, entry_of_token, q_start, slot_ids},
-             ld, dt_col, heads * P + 2 * groups * N, heads, P, N, groups};
-  const dim3 grid(heads, num_entries, (P + kScanCols - 1) / kScanCols);
-  const dim3 block(kScanSlices * kScanCols);
+             ld, dt_col, heads * P + 2 * groups * N, heads, P, N, groups,
+             chunks, entry_chunks, chunk_state, chunk_decay};
   const int ni = (N + kScanSlices - 1) / kScanSlices;
-  if (ni <= 2) hipLaunchKernelGGL(ssm_scan_kernel<2>, grid, block, 0, stream, a);
-  else if (ni <= 4) hipLaunchKernelGGL(ssm_scan_kernel<4>, grid, block, 0, stream, a);
-  else if (ni <= 8) hipLaunchKernelGGL(ssm_scan_kernel<8>, grid, block, 0, stream, a);
-  else if (ni <= 16) hipLaunchKernelGGL(ssm_scan_kernel<16>, grid, block, 0, stream, a);
-  else hipLaunchKernelGGL(ssm_scan_kernel<32>, grid, block, 0, stream, a);
+  if (ni <= 2) launch_scan<2>(a, num_entries, num_chunks, stream);
+  else if (ni <= 4) launch_scan<4>(a, num_entries, num_chunks, stream);
+  else if (ni <= 8) launch_scan<8>(a, num_entries, num_chunks, stream);
+  else if (ni <= 16) launch_scan<16>(a, num_entries, num_chunks, stream);
+  else launch_scan<32>(a, num_entries, num_chunks, stream);
   TS_CHECK_LAUNCH("ssm_scan");
   return 0;
 }

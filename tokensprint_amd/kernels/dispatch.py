@@ -78,6 +78,13 @@ class Dispatch:
     cooperative_workgroups: int = 512
     per_wave_workgroups: int = 4096
 
+    # ---- state-space recurrence.  A step whose longest portion has more tokens than this
+    # is cut into chunks of 64 tokens that run side by side (three launches, twice the
+    # arithmetic); below it every entry is walked whole by one launch.  At 64 heads of 64
+    # columns and 128 state rows a walked token costs about 0.3 us, a chunked portion about
+    # as much as 130 walked tokens whatever its length.
+    scan_whole_tokens: int = 128
+
 
 #: what each table was measured on -> the table
 MEASURED: dict[str, Dispatch] = {

@@ -1058,9 +1058,27 @@ class HipOps:
         self._check_state("recurrent state", state, (heads, N, vdim))
         pos, eot, qs, slots = self._batch_ptrs(batch, T)
         y = torch.empty(T, inner, dtype=torch.float32, device=self.device)
+        # a step with a long portion runs its entries in chunks side by side (the lists are
+        # the step's: every recurrent layer of the model uses the same)
+        chunks = entry_chunks = scratch = decays = None
+        num_chunks = 0
+        if batch.max_q_len > self.dispatch.scan_whole_tokens:
+            if "scan_chunks" not in batch.plans:
+                size, rows, firsts, t0 = self.lib.ts_ssm_scan_chunk(), [], [0], 0
+                for e, n in enumerate(batch.q_lens):
+                    rows += [(t0 + c, min(t0 + c + size, t0 + n), e) for c in range(0, n, size)]
+                    firsts.append(len(rows))
+                    t0 += n
+                batch.plans["scan_chunks"] = (self._upload_ints(rows), self._upload_ints(firsts),
+                                              len(rows))
+            chunks, entry_chunks, num_chunks = batch.plans["scan_chunks"]
+            scratch = torch.empty(num_chunks, heads, N, vdim, dtype=torch.float32,
+                                  device=self.device)
+            decays = torch.empty(num_chunks, heads, dtype=torch.float32, device=self.device)
         self._call(self.lib.ts_ssm_scan, _ptr(xbc), _ptr(proj), proj.shape[1], dt_col,
                    _ptr(dt_bias), _ptr(a_log), _ptr(d_skip), _ptr(state), _ptr(y), pos, eot, qs,
-                   slots, T, batch.num_entries, heads, vdim, N, groups, self._stream())
+                   slots, T, batch.num_entries, heads, vdim, N, groups, _ptr(chunks),
+                   _ptr(entry_chunks), num_chunks, _ptr(scratch), _ptr(decays), self._stream())
         return y
 
     def gated_group_norm(self, y, proj, norm_w, groups, eps, out_dtype):
@@ -1109,27 +1127,22 @@ class HipOps:
                    self._stream())
         return cq
 
-    def latent_query(self, q, w_uk, batch, *, heads, dim, rot_dim, kv_rank, freqs, rot_dims):
-        """q [T, heads*(dim+rot_dim)] float32 -> [T, heads, kv_rank+rot_dim] float32: the
-        unrotated part carried through U_k (w_uk [heads*dim, kv_rank]) into the latent's
-        space, the rotated part rotated at the token's position."""
-        self._check("q", q, torch.float32, ndim=2)
-        T = q.shape[0]
-        if q.shape[1] != heads * (dim + rot_dim):
-            raise ValueError("latent_query: q rows do not fit heads * (dim + rot_dim)")
-        self._check("U_k", w_uk, self._FLOATS, shape=(heads * dim, kv_rank))
-        self._check("frequencies", freqs, torch.float32, shape=(rot_dims // 2,))
-        self._check("positions", batch.positions, torch.int32, shape=(T,))
-        out = torch.empty(T, heads, kv_rank + rot_dim, dtype=torch.float32, device=self.device)
-        self._call(self.lib.ts_latent_query, _ptr(q), _ptr(w_uk), _TYPE_CODE[w_uk.dtype],
-                   _ptr(freqs), _ptr(batch.positions), _ptr(out), T, heads, dim, rot_dim, kv_rank,
-                   rot_dims, self._stream())
-        return out
+    def rotate_interleaved_inplace(self, x, positions, freqs, dims, offset=0):
+        """x [T, heads, width]: the pairs (offset + 2i, offset + 2i + 1), i < dims / 2, of
+        every head's vector turned by positions[t] * freqs[i], in place."""
+        self._check("x", x, self._FLOATS, ndim=3)
+        T, heads, width = x.shape
+        self._check("positions", positions, torch.int32, shape=(T,))
+        self._check("frequencies", freqs, torch.float32, shape=(dims // 2,))
+        if dims % 2 or offset < 0 or offset + dims > width:
+            raise ValueError(f"rotate_interleaved: {dims} dimensions from {offset} of {width}")
+        self._call(self.lib.ts_rotate_interleaved, _ptr(x), _TYPE_CODE[x.dtype], _ptr(positions),
+                   _ptr(freqs), T, heads, width, offset, dims, self._stream())
 
     def latent_attention(self, qa, batch, table, cache, *, heads, kv_rank, rot_dim, scale,
-                         window):
+                         window, out_dtype=torch.float32):
         """Softmax attention of qa [T, heads, kv_rank+rot_dim] (float32) over the latent
-        pages -> sum_t p_t c_t, float32 [T, heads, kv_rank]."""
+        pages -> sum_t p_t c_t, [T, heads, kv_rank] in `out_dtype`."""
         dl = kv_rank + rot_dim
         self._check("qa", qa, torch.float32, ndim=3)
         T = qa.shape[0]
@@ -1137,23 +1150,10 @@ class HipOps:
             raise ValueError("latent_attention: query shape does not fit")
         self._check_latent(cache, table, batch, dl)
         pos, eot, _, _ = self._batch_ptrs(batch, T)
-        out = torch.empty(T, heads, kv_rank, dtype=torch.float32, device=self.device)
+        out = torch.empty(T, heads, kv_rank, dtype=out_dtype, device=self.device)
         self._call(self.lib.ts_latent_attention, _ptr(qa), _ptr(cache.k_pages),
-                   _TYPE_CODE[cache.k_pages.dtype], _ptr(out), pos, eot, _ptr(table),
+                   _TYPE_CODE[cache.k_pages.dtype], _ptr(out), _TYPE_CODE[out_dtype], pos, eot,
+                   _ptr(table),
                    table.shape[1], cache.page_size, T, heads, kv_rank, rot_dim,
                    int(window) if window else 0, c_float(scale), self._stream())
-        return out
-
-    def head_linear(self, x, weight, heads, out_dtype):
-        """x [T, heads, in] float32, weight [heads*rows, in] -> [T, heads*rows]: each head's
-        rows of the weight applied to that head's vector."""
-        self._check("x", x, torch.float32, ndim=3)
-        T, H, n_in = x.shape
-        self._check("weight", weight, self._FLOATS, ndim=2)
-        if H != heads or weight.shape[1] != n_in or weight.shape[0] % heads:
-            raise ValueError("head_linear: shapes do not fit")
-        rows = weight.shape[0] // heads
-        out = torch.empty(T, heads * rows, dtype=out_dtype, device=self.device)
-        self._call(self.lib.ts_head_linear, _ptr(x), _ptr(weight), _TYPE_CODE[weight.dtype],
-                   _ptr(out), _TYPE_CODE[out_dtype], T, heads, rows, n_in, self._stream())
         return out

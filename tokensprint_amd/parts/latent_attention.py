@@ -9,8 +9,13 @@ rotated like k_r)
     out_j(i)      = U_v,j  sum_t softmax_t(score_j(i, t)) c_t
 
 and neither keys nor values are ever expanded: queries are carried into the latent's space
-before attention, and its output back out of it afterwards.  Queries come through a latent
-of their own (down, RMS norm, up).  A window W lets position i see positions i-W+1..i.
+before attention, and its output back out of it afterwards.  Both steps are folded into the
+weights when they are loaded (products taken in float64, rounded once to the run's dtype):
+the query up-projection becomes [U_k,j^T U_q,j ; U_q,j's rotated rows] per head, a plain
+product from the query latent straight to q', and the output projection becomes
+W_o,j U_v,j per head, a plain product from the attention's latent-space result to the
+model width.  Queries come through a latent of their own (down, RMS norm, up).  A window W
+lets position i see positions i-W+1..i.
 """
 
 from __future__ import annotations
@@ -37,7 +42,7 @@ class LatentAttention(Mixer):
         if self.position.dims > self.rot_dim:
             raise ValueError(f"{self.prefix}: the rotation covers {self.position.dims} "
                              f"dimensions, the rotated part has {self.rot_dim}")
-        self.w_down = self.w_uq = self.w_uk = self.w_uv = self.w_o = None
+        self.w_down = self.w_query = self.w_out = None
         self.q_norm = self.kv_norm = None
 
     def tensors(self):
@@ -60,8 +65,15 @@ class LatentAttention(Mixer):
             raise ValueError(f"{pre}: the two down projections are stored in different dtypes")
         self.w_down = torch.cat([dq, dkv], dim=0).contiguous()
         self.q_norm, self.kv_norm = get(pre + "dq.norm"), get(pre + "dkv.norm")
-        self.w_uq, self.w_uk, self.w_uv = get(pre + "uq"), get(pre + "uk"), get(pre + "uv")
-        self.w_o = get(pre + "o")
+        H, dn, dr, R, dv = self.heads, self.dim, self.rot_dim, self.kv_rank, self.vdim
+        uq, uk, uv, wo = get(pre + "uq"), get(pre + "uk"), get(pre + "uv"), get(pre + "o")
+        uq64 = uq.double().view(H, dn + dr, self.q_rank)
+        carried = torch.einsum("hdr,hdq->hrq", uk.double().view(H, dn, R), uq64[:, :dn])
+        self.w_query = torch.cat([carried, uq64[:, dn:]], dim=1) \
+            .reshape(H * (R + dr), self.q_rank).to(uq.dtype).contiguous()
+        self.w_out = torch.einsum("whv,hvr->whr", wo.double().view(-1, H, dv),
+                                  uv.double().view(H, dv, R)) \
+            .reshape(-1, H * R).to(wo.dtype).contiguous()
 
     def cache_need(self):
         return PagedLatentNeed(self.kv_rank + self.rot_dim, self.window)
@@ -79,12 +91,11 @@ class LatentAttention(Mixer):
                                 kv_rank=self.kv_rank, rot_dim=self.rot_dim, q_norm=self.q_norm,
                                 kv_norm=self.kv_norm, eps=self.eps, freqs=freqs,
                                 rot_dims=rot_dims, out_dtype=self.ctx.dtype)
-        q = ops.linear(cq, self.w_uq, torch.float32)
-        qa = ops.latent_query(q, self.w_uk, batch, heads=self.heads, dim=self.dim,
-                              rot_dim=self.rot_dim, kv_rank=self.kv_rank, freqs=freqs,
-                              rot_dims=rot_dims)
+        T = h.shape[0]
+        qa = ops.linear(cq, self.w_query, torch.float32).view(T, self.heads,
+                                                              self.kv_rank + self.rot_dim)
+        ops.rotate_interleaved_inplace(qa, batch.positions, freqs, rot_dims, offset=self.kv_rank)
         ol = ops.latent_attention(qa, batch, table, cache, heads=self.heads,
                                   kv_rank=self.kv_rank, rot_dim=self.rot_dim, scale=self.scale,
-                                  window=self.window)
-        o = ops.head_linear(ol, self.w_uv, self.heads, self.ctx.dtype)
-        return ops.linear(o, self.w_o, torch.float32)
+                                  window=self.window, out_dtype=self.ctx.dtype)
+        return ops.linear(ol.view(T, self.heads * self.kv_rank), self.w_out, torch.float32)

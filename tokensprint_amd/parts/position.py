@@ -68,6 +68,6 @@ class InterleavedRotation(PositionEncoding):
         return []
 
     def apply(self, q, k, positions):
-        self.ops.rotate_interleaved_inplace(q, positions, self.freqs, self.dims)
+        self.ops.rotate_interleaved_inplace(q, positions, self.freqs, self.dims, offset=0)
         if k is not None:
-            self.ops.rotate_interleaved_inplace(k, positions, self.freqs, self.dims)
+            self.ops.rotate_interleaved_inplace(k, positions, self.freqs, self.dims, offset=0)
