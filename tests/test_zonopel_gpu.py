@@ -251,25 +251,31 @@ def test_latent_attention_kernels(gpu_device, cache_dtype, heads, dim, rot_dim, 
         close(qa, qb)
         kw = dict(heads=heads, kv_rank=kv_rank, rot_dim=rot_dim, scale=0.2, window=window)
         ol = REF.latent_attention(qb, batch, table, ref_view, **kw)
-        close(ops.latent_attention(qb, batch, table, scene.view, **kw), ol, **tol)
+        # (bfloat16 pages take the matrix-core kernel, which rounds queries and softmax
+        # weights to bfloat16: scores of standard deviation 5 move by a few hundredths)
+        loose = dict(rtol=6e-2, atol=6e-2)
+        close(ops.latent_attention(qb, batch, table, scene.view, **kw), ol,
+              **(tol if cache_dtype == torch.float32 else loose))
         got = ops.latent_attention(qb, batch, table, scene.view, out_dtype=torch.bfloat16, **kw)
         assert got.dtype == torch.bfloat16
-        close(got, ol, rtol=2e-2, atol=2e-2)
+        close(got, ol, **loose)
 
 
+@pytest.mark.parametrize("cache_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("window", [None, 20, 64, 65])
 @pytest.mark.parametrize("decode", [False, True])
-def test_one_key_stands_out(gpu_device, window, decode):
+def test_one_key_stands_out(gpu_device, window, decode, cache_dtype):
     """Rows of the pages are small noise but for one, which the query points at: the
     result is that row if the query can see it (far back without a window, or the first
     token inside one) and noise if it is the first token outside."""
     ops = load_hip_ops(gpu_device)
-    heads, kv_rank, rot_dim, page = 2, 16, 4, 8
+    heads, kv_rank, rot_dim, page = 2, 16, 8, 8      # (bfloat16 pages: the matrix-core kernel)
     dl, T = kv_rank + rot_dim, 301
     for where in ("inside", "outside"):
         if window is None and where == "outside":
             continue
-        scene = Scene(gpu_device, PagedLatentNeed(dl, None), page, 1, num_pages=45)
+        scene = Scene(gpu_device, PagedLatentNeed(dl, None), page, 1, dtype=cache_dtype,
+                      num_pages=45)
         batch = scene.step([T])
         if decode:
             batch = BatchBuilder(gpu_device, 1).build(
@@ -281,7 +287,8 @@ def test_one_key_stands_out(gpu_device, window, decode):
         rows[target] = direction * 3.0
         table = batch.tables[0][0].cpu()
         pos = torch.arange(T)
-        scene.view.k_pages[table[pos // page].long(), pos % page] = rows.to(gpu_device)
+        rows = rows.to(cache_dtype).float()
+        scene.view.k_pages[table[pos // page].long(), pos % page] = rows.to(cache_dtype).to(gpu_device)
         n = batch.num_tokens
         qa = torch.zeros(n, heads, dl)
         qa[-1] = direction * 40.0
@@ -290,7 +297,7 @@ def test_one_key_stands_out(gpu_device, window, decode):
                                    window=window)[-1].cpu()
         if where == "inside":
             torch.testing.assert_close(out, rows[target, :kv_rank].expand(heads, -1),
-                                       rtol=1e-3, atol=1e-3)
+                                       rtol=1e-3, atol=1e-3 if cache_dtype == torch.float32 else 2e-2)
         else:
             assert out.abs().max() < 0.1
 

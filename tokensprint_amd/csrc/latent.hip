@@ -237,3 +237,261 @@ extern "C" int ts_latent_attention(const float* qa, const void* pages, int cache
   return 0;
 }
 
+
+// ---------------------------------------------------------------- attention on the matrix cores
+// bfloat16 pages.  A tile is 16 consecutive rows of the step's (token, head) rows that
+// belong to one entry: every head reads the same cached rows, so a decode step's token is
+// one tile of its heads, and a prompt's tile a few tokens with all their heads.  One
+// wavefront per (tile, share of the keys):
+//     S^T = K Q'^T        v_mfma_f32_16x16x32_bf16, reduction over the latent row
+//     O^T += C^T P^T      the same instruction, reduction over 32 keys
+// Lane (r, g) = (lane % 16, lane / 16) owns query row r: its scores come out as
+// S^T[key 4g + t][row r], which is, in place, its part of the second product's B operand;
+// its softmax statistics are shared with lanes r + 16, r + 32, r + 48; its part of O^T is
+// [columns 16 db + 4g + t][row r], so rescaling needs nothing from other lanes.
+// Keys are walked in blocks of 32 at absolute multiples of 32.  Where a step has few
+// tiles, a tile's keys are shared out in runs of `keys_per_split` over several wavefronts,
+// whose unnormalised results and statistics a second kernel merges.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_l;
+
+struct LatentMfmaArgs {
+  const float* qa;          // [rows, dl], rows = tokens * heads
+  const bf16_t* pages;      // [pages, page_size, dl]
+  void* out;                // [rows, kv_rank]
+  const int* tiles;         // [num_tiles, 3]: first row, rows (1..16), entry
+  const int* positions;     // [tokens]
+  const int* table;
+  float* part_o;            // [num_tiles, splits, 16, kv_rank]
+  float* part_ml;           // [num_tiles, splits, 16, 2]
+  int table_width, page_size, heads, kv_rank, rot_dim, window, keys_per_split, splits;
+  float scale;
+};
+
+constexpr int kLatentPad = 8;     // elements between staged rows: operand reads spread over banks
+
+// The wavefronts of a workgroup (four where keys are not shared out, else one) take
+// consecutive tiles of one entry and walk the union of their keys together: each block of
+// 32 cached rows is staged in LDS once by all of them (16-byte loads, rows that are not
+// there as zeros), and both operands come from there: the K operand as 16 bytes of a row,
+// the C^T operand as eight 2-byte reads of a column.  A tile with no rows only helps load.
+template <int KS, int DB, typename TO>
+__global__ __launch_bounds__(4 * kWave) void latent_attention_mfma_kernel(LatentMfmaArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const int dl = a.kv_rank + a.rot_dim, P = a.page_size;
+  const int stride = dl + kLatentPad;
+  bf16_t* k_s = (bf16_t*)lds_raw;                         // [32][stride]
+  int* krow_s = (int*)(lds_raw + (size_t)32 * stride * sizeof(bf16_t));   // [32]
+  const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave, r = lane % 16, g = lane / 16;
+  const int tile0 = blockIdx.x * waves, tile = tile0 + wave, split = blockIdx.y;
+  const int row0 = a.tiles[3 * tile], nrows = a.tiles[3 * tile + 1];
+  const int* tab = a.table + (int64_t)a.tiles[3 * tile0 + 2] * a.table_width;
+  const bool row_ok = r < nrows;
+  const int my_row = row0 + max(0, min(r, nrows - 1));
+  const int pos_r = a.positions[my_row / a.heads];
+  const int lo_r = a.window > 0 ? max(0, pos_r - a.window + 1) : 0;
+  // the keys of the whole workgroup: from the first tile's first token to the last token
+  const int pos_first = a.positions[a.tiles[3 * tile0] / a.heads];
+  const int lo_t = a.window > 0 ? max(0, pos_first - a.window + 1) : 0;
+  int hi_t = pos_first;
+  for (int w = 0; w < waves; ++w) {
+    const int n = a.tiles[3 * (tile0 + w) + 1];
+    if (n > 0) hi_t = max(hi_t, a.positions[(a.tiles[3 * (tile0 + w)] + n - 1) / a.heads]);
+  }
+  const int k_begin = (lo_t / 32) * 32 + split * a.keys_per_split;
+  const int k_end = min(k_begin + a.keys_per_split, hi_t + 1);
+
+  bf16x8_l q[KS];
+  const float* qr = a.qa + (int64_t)my_row * dl;
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    const int d0 = 32 * s + 8 * g;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) q[s][j] = (d0 + j < dl) ? (__bf16)qr[d0 + j] : (__bf16)0.f;
+  }
+  f32x4_l o[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) o[db] = f32x4_l{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int parts = dl / 8;
+
+  for (int kb = k_begin; kb < k_end; kb += 32) {
+    __syncthreads();                      // the block before has been used by everyone
+    for (int c = threadIdx.x; c < 32 * parts; c += blockDim.x) {
+      const int key = c / parts, part = c % parts;
+      const int j = kb + key;
+      int page = -1;
+      if (j >= lo_t && j <= hi_t) page = tab[j / P];
+      const int row = page >= 0 ? page * P + j % P : -1;
+      bf16x8_l v;
+      if (row >= 0) v = *(const bf16x8_l*)(a.pages + (int64_t)row * dl + part * 8);
+      else {
+#pragma unroll
+        for (int j8 = 0; j8 < 8; ++j8) v[j8] = (__bf16)0.f;
+      }
+      *(bf16x8_l*)(k_s + key * stride + part * 8) = v;
+      if (part == 0) krow_s[key] = row;
+    }
+    __syncthreads();
+    f32x4_l st[2];
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      const bf16_t* kr = k_s + (16 * blk + r) * stride;
+      st[blk] = f32x4_l{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const int d0 = 32 * s + 8 * g;
+        if (32 * s < dl) {
+          bf16x8_l kop;
+          if (d0 + 8 <= dl) kop = *(const bf16x8_l*)(kr + d0);
+          else {
+#pragma unroll
+            for (int j8 = 0; j8 < 8; ++j8) kop[j8] = (__bf16)0.f;
+          }
+          st[blk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, q[s], st[blk], 0, 0, 0);
+        }
+      }
+    }
+    float sc[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int blk = e / 4, t = e % 4;
+      const int key = kb + 16 * blk + 4 * g + t;
+      const bool vis = row_ok && krow_s[16 * blk + 4 * g + t] >= 0 && key <= pos_r && key >= lo_r;
+      sc[e] = vis ? st[blk][t] * a.scale : -INFINITY;
+      mx = fmaxf(mx, sc[e]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    const float m_new = fmaxf(m, mx);
+    const float corr = m_new == -INFINITY ? 1.f : expf(m - m_new);
+    bf16x8_l pv;
+    float psum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float p = sc[e] == -INFINITY ? 0.f : expf(sc[e] - m_new);
+      psum += p;
+      pv[e] = (__bf16)p;
+    }
+    psum += __shfl_xor(psum, 16, kWave);
+    psum += __shfl_xor(psum, 32, kWave);
+    l = l * corr + psum;
+    m = m_new;
+    const bf16_t* vcol = k_s + (4 * g) * stride + r;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      if (16 * db < a.kv_rank) {
+        bf16x8_l vop;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          vop[e] = vcol[(16 * (e / 4) + e % 4) * stride + 16 * db];
+        o[db] = o[db] * corr;
+        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pv, o[db], 0, 0, 0);
+      }
+    }
+  }
+  if (a.splits == 1) {
+    if (!row_ok) return;
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    TO* orow = (TO*)a.out + (int64_t)my_row * a.kv_rank;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int d = 16 * db + 4 * g + t;
+        if (d < a.kv_rank) orow[d] = from_f32<TO>(o[db][t] * inv);
+      }
+    return;
+  }
+  const int64_t slot = ((int64_t)tile * a.splits + split) * 16 + r;
+  float* po = a.part_o + slot * a.kv_rank;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int d = 16 * db + 4 * g + t;
+      if (d < a.kv_rank) po[d] = o[db][t];
+    }
+  if (g == 0) {
+    a.part_ml[2 * slot] = m;
+    a.part_ml[2 * slot + 1] = l;
+  }
+}
+
+// One workgroup per (tile, row): the shares' results weighted by exp(m_s - max m) and
+// divided by the summed weights of their l, shares in index order.
+template <typename TO>
+__global__ __launch_bounds__(128) void latent_attention_merge_kernel(LatentMfmaArgs a) {
+  const int tile = blockIdx.x, r = blockIdx.y;
+  if (r >= a.tiles[3 * tile + 1]) return;
+  const int64_t base = (int64_t)tile * a.splits * 16 + r;
+  float mx = -INFINITY;
+  for (int s = 0; s < a.splits; ++s) mx = fmaxf(mx, a.part_ml[2 * (base + 16 * s)]);
+  float total = 0.f;
+  for (int s = 0; s < a.splits; ++s) {
+    const float ms = a.part_ml[2 * (base + 16 * s)];
+    if (ms != -INFINITY) total += a.part_ml[2 * (base + 16 * s) + 1] * expf(ms - mx);
+  }
+  const float inv = total > 0.f ? 1.0f / total : 0.f;
+  TO* orow = (TO*)a.out + (int64_t)(a.tiles[3 * tile] + r) * a.kv_rank;
+  for (int d = threadIdx.x; d < a.kv_rank; d += blockDim.x) {
+    float acc = 0.f;
+    for (int s = 0; s < a.splits; ++s) {
+      const float ms = a.part_ml[2 * (base + 16 * s)];
+      if (ms != -INFINITY) acc = fmaf(a.part_o[(base + 16 * s) * a.kv_rank + d], expf(ms - mx), acc);
+    }
+    orow[d] = from_f32<TO>(acc * inv);
+  }
+}
+
+template <int KS, int DB>
+static int launch_latent_mfma(const LatentMfmaArgs& a, int num_tiles, int waves, int out_type,
+                              hipStream_t stream) {
+  const int dl = a.kv_rank + a.rot_dim;
+  const size_t lds = (size_t)32 * (dl + kLatentPad) * sizeof(bf16_t) + 32 * sizeof(int);
+  TS_DISPATCH_TYPE(out_type, TO, {
+    hipLaunchKernelGGL((latent_attention_mfma_kernel<KS, DB, TO>),
+                       dim3(num_tiles / waves, a.splits), dim3(waves * kWave), lds, stream, a);
+    if (a.splits > 1)
+      hipLaunchKernelGGL(latent_attention_merge_kernel<TO>, dim3(num_tiles, 16), dim3(128), 0,
+                         stream, a);
+  });
+  return 0;
+}
+
+// 1 if the matrix-core kernel serves these sizes (bfloat16 pages are the caller's to check).
+extern "C" int ts_latent_attention_mfma_fits(int kv_rank, int rot_dim) {
+  const int dl = kv_rank + rot_dim;
+  return dl % 8 == 0 && dl <= 640 && kv_rank <= 512;
+}
+
+// `tiles` comes in groups of `waves` (1 or 4) tiles of one entry, a group's last tiles
+// possibly empty (0 rows); `num_tiles` counts them all.
+extern "C" int ts_latent_attention_mfma(const float* qa, const void* pages, void* out,
+                                        int out_type, const int* tiles, int num_tiles, int waves,
+                                        const int* positions, const int* table, int table_width,
+                                        int page_size, int heads, int kv_rank, int rot_dim,
+                                        int window, float scale, int keys_per_split, int splits,
+                                        float* part_o, float* part_ml, hipStream_t stream) {
+  if (num_tiles <= 0) return 0;
+  if (!ts_latent_attention_mfma_fits(kv_rank, rot_dim) || heads <= 0 || page_size <= 0)
+    TS_FAIL("latent_attention_mfma: sizes kv_rank=%d rot_dim=%d are not served", kv_rank, rot_dim);
+  if (splits < 1 || keys_per_split < 32 || keys_per_split % 32)
+    TS_FAIL("latent_attention_mfma: bad split of the keys (%d runs of %d)", splits, keys_per_split);
+  if (splits > 1 && (!part_o || !part_ml)) TS_FAIL("latent_attention_mfma: no scratch for the shares");
+  if ((waves != 1 && waves != 4) || num_tiles % waves)
+    TS_FAIL("latent_attention_mfma: %d tiles in groups of %d", num_tiles, waves);
+  if (((uintptr_t)pages & 15) != 0) TS_FAIL("latent_attention_mfma: pages must start on 16 bytes");
+  LatentMfmaArgs a{qa, (const bf16_t*)pages, out, tiles, positions, table, part_o, part_ml,
+                   table_width, page_size, heads, kv_rank, rot_dim, window, keys_per_split, splits,
+                   scale};
+  const int dl = kv_rank + rot_dim;
+  int rc;
+  if (dl <= 96 && kv_rank <= 64) rc = launch_latent_mfma<3, 4>(a, num_tiles, waves, out_type, stream);
+  else if (dl <= 320 && kv_rank <= 256) rc = launch_latent_mfma<10, 16>(a, num_tiles, waves, out_type, stream);
+  else rc = launch_latent_mfma<20, 32>(a, num_tiles, waves, out_type, stream);
+  if (rc) return rc;
+  TS_CHECK_LAUNCH("latent_attention_mfma");
+  return 0;
+}

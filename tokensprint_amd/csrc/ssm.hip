@@ -142,10 +142,9 @@ extern "C" int ts_conv_silu(const float* proj, int ld, int col, int channels, in
 // ---------------------------------------------------------------- recurrence
 // Per head h (group g): d = softplus(dt + dt_bias[h]), a = exp(-exp(A_log[h]) d),
 //   S <- a S + (d B_g) x_h^T   (S: N x P),   y_h = S^T C_g + D[h] x_h.
-// A workgroup serves one (run of tokens, head, 32 columns of P): thread (p, s) keeps rows
-// s, s + 8, ... of column p in registers, walks the tokens in order and adds the eight
-// slices of a column's dot product through the wavefront.  The operands of the next token
-// are fetched while the current one is computed.
+// A workgroup serves one (run of tokens, head, 64 columns of P): a thread keeps eight-strided
+// rows of four columns in registers, walks the tokens in order and adds the eight slices of
+// a column's dot product through the wavefront.
 //
 // Steps of few tokens per entry walk each entry whole (kScanWhole).  A long portion is cut
 // into chunks of 64 tokens that run side by side, in three launches: every chunk's
@@ -170,16 +169,30 @@ struct ScanArgs {
 };
 
 constexpr int kScanSlices = 8;
-constexpr int kScanCols = 32;
+constexpr int kScanCols = 32;              // columns of a workgroup of the combine kernel
 constexpr int kScanWhole = 0, kScanLocal = 1, kScanOutput = 2;
+constexpr int kScanThreads = 128;          // the walking kernel: 8 slices x 16 groups of columns
+constexpr int kScanPerThread = 4;          // columns a thread owns
+constexpr int kScanBlockCols = kScanThreads / kScanSlices * kScanPerThread;   // 64
+constexpr int kScanStage = 16;             // tokens staged in LDS at a time
 
+// Thread (cg, s) = (tid / 8, tid % 8) keeps rows s, s + 8, ... of four columns in registers.
+// Sixteen tokens' operands (B, C, the workgroup's columns of x, the step and the decay,
+// computed once a token) are staged in LDS by all threads together, then walked in order:
+// a token costs a thread 2 NI + 3 LDS reads for 8 NI multiply-adds.
 template <int NI, int MODE>
-__global__ __launch_bounds__(kScanSlices* kScanCols) void ssm_scan_kernel(ScanArgs a) {
+__global__ __launch_bounds__(kScanThreads) void ssm_scan_kernel(ScanArgs a) {
+  extern __shared__ float lds[];
+  const int N = a.N;
+  float* B_s = lds;                                  // [stage][N]
+  float* C_s = B_s + kScanStage * N;                 // [stage][N]
+  float* x_s = C_s + kScanStage * N;                 // [stage][64]
+  float* d_s = x_s + kScanStage * kScanBlockCols;    // [stage]: step size
+  float* a_s = d_s + kScanStage;                     // [stage]: decay
   const int h = blockIdx.x;
-  const int p = blockIdx.z * kScanCols + threadIdx.x / kScanSlices;
-  const int s = threadIdx.x % kScanSlices;
-  const bool live = p < a.P;
-  const int pc = live ? p : a.P - 1;      // idle columns shadow the last one and store nothing
+  const int s = threadIdx.x % kScanSlices, cg = threadIdx.x / kScanSlices;
+  const int col0 = blockIdx.z * kScanBlockCols;
+  const int p0 = col0 + cg * kScanPerThread;
   const int g = h / (a.heads / a.groups);
   int first, end, e;
   if (MODE == kScanWhole) {
@@ -192,71 +205,89 @@ __global__ __launch_bounds__(kScanSlices* kScanCols) void ssm_scan_kernel(ScanAr
     e = a.chunks[3 * blockIdx.y + 2];
   }
   const int inner = a.heads * a.P;
-  const int N = a.N;
   float* st = MODE == kScanWhole
       ? a.state + ((int64_t)a.b.slot_ids[e] * a.heads + h) * N * a.P
       : a.chunk_state + ((int64_t)blockIdx.y * a.heads + h) * N * a.P;
-  float S[NI];
+  float S[NI][kScanPerThread];
   const bool fresh = MODE == kScanLocal || (MODE == kScanWhole && a.b.positions[first] == 0);
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
     const int n = s + kScanSlices * i;
-    S[i] = (!fresh && n < N) ? st[(int64_t)n * a.P + pc] : 0.f;
+#pragma unroll
+    for (int c = 0; c < kScanPerThread; ++c)
+      S[i][c] = (!fresh && n < N && p0 + c < a.P) ? st[(int64_t)n * a.P + p0 + c] : 0.f;
   }
   const float decay_rate = -expf(a.a_log[h]);
   const float bias = a.dt_bias[h], skip = a.d_skip[h];
   const int b_col = inner + g * N, c_col = inner + a.groups * N + g * N;
-
-  float nB[NI], nC[NI], nx, ndt;
-  auto fetch = [&](int t) {
-    const float* row = a.xbc + (int64_t)t * a.channels;
-    nx = row[h * a.P + pc];
-    ndt = a.proj[(int64_t)t * a.ld + a.dt_col + h];
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      const int n = s + kScanSlices * i;
-      nB[i] = n < N ? row[b_col + n] : 0.f;
-      if (MODE != kScanLocal) nC[i] = n < N ? row[c_col + n] : 0.f;
-    }
-  };
-  if (first < end) fetch(first);
   float total_decay = 1.f;
-  for (int t = first; t < end; ++t) {
-    float B[NI], C[NI];
-    const float x = nx, dt_raw = ndt;
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      B[i] = nB[i];
-      if (MODE != kScanLocal) C[i] = nC[i];
+
+  for (int t0 = first; t0 < end; t0 += kScanStage) {
+    const int nt = min(kScanStage, end - t0);
+    __syncthreads();                                  // the stage before has been walked
+    for (int i = threadIdx.x; i < nt * N; i += kScanThreads) {
+      const float* row = a.xbc + (int64_t)(t0 + i / N) * a.channels;
+      B_s[i] = row[b_col + i % N];
+      if (MODE != kScanLocal) C_s[i] = row[c_col + i % N];
     }
-    if (t + 1 < end) fetch(t + 1);
-    const float d = softplus_f(dt_raw + bias);
-    const float decay = expf(decay_rate * d);
-    const float dx = d * x;
-    if (MODE == kScanLocal) {
-      total_decay *= decay;
-#pragma unroll
-      for (int i = 0; i < NI; ++i) S[i] = fmaf(decay, S[i], B[i] * dx);
-      continue;
+    for (int i = threadIdx.x; i < nt * kScanBlockCols; i += kScanThreads) {
+      const int tt = i / kScanBlockCols, c = i % kScanBlockCols;
+      x_s[i] = col0 + c < a.P ? a.xbc[(int64_t)(t0 + tt) * a.channels + h * a.P + col0 + c] : 0.f;
     }
-    float acc = 0.f;
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      S[i] = fmaf(decay, S[i], B[i] * dx);
-      acc = fmaf(S[i], C[i], acc);
+    if (threadIdx.x < nt) {
+      const float d = softplus_f(a.proj[(int64_t)(t0 + threadIdx.x) * a.ld + a.dt_col + h] + bias);
+      d_s[threadIdx.x] = d;
+      a_s[threadIdx.x] = expf(decay_rate * d);
     }
-    acc += __shfl_xor(acc, 1, kWave);
-    acc += __shfl_xor(acc, 2, kWave);
-    acc += __shfl_xor(acc, 4, kWave);
-    if (s == 0 && live) a.y[(int64_t)t * inner + h * a.P + p] = fmaf(skip, x, acc);
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float d = d_s[tt], decay = a_s[tt];
+      float dx[kScanPerThread], x[kScanPerThread], acc[kScanPerThread];
+#pragma unroll
+      for (int c = 0; c < kScanPerThread; ++c) {
+        x[c] = x_s[tt * kScanBlockCols + cg * kScanPerThread + c];
+        dx[c] = d * x[c];
+        acc[c] = 0.f;
+      }
+      if (MODE == kScanLocal) {
+        total_decay *= decay;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+          const int n = s + kScanSlices * i;
+          const float Bv = n < N ? B_s[tt * N + n] : 0.f;
+#pragma unroll
+          for (int c = 0; c < kScanPerThread; ++c) S[i][c] = fmaf(decay, S[i][c], Bv * dx[c]);
+        }
+        continue;
+      }
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int n = s + kScanSlices * i;
+        const float Bv = n < N ? B_s[tt * N + n] : 0.f;
+        const float Cv = n < N ? C_s[tt * N + n] : 0.f;
+#pragma unroll
+        for (int c = 0; c < kScanPerThread; ++c) {
+          S[i][c] = fmaf(decay, S[i][c], Bv * dx[c]);
+          acc[c] = fmaf(S[i][c], Cv, acc[c]);
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < kScanPerThread; ++c) {
+        acc[c] += __shfl_xor(acc[c], 1, kWave);
+        acc[c] += __shfl_xor(acc[c], 2, kWave);
+        acc[c] += __shfl_xor(acc[c], 4, kWave);
+        if (s == 0 && p0 + c < a.P)
+          a.y[(int64_t)(t0 + tt) * inner + h * a.P + p0 + c] = fmaf(skip, x[c], acc[c]);
+      }
+    }
   }
   if (MODE == kScanOutput) return;
-  if (live) {
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      const int n = s + kScanSlices * i;
-      if (n < N) st[(int64_t)n * a.P + p] = S[i];
-    }
+  for (int i = 0; i < NI; ++i) {
+    const int n = s + kScanSlices * i;
+#pragma unroll
+    for (int c = 0; c < kScanPerThread; ++c)
+      if (n < N && p0 + c < a.P) st[(int64_t)n * a.P + p0 + c] = S[i][c];
   }
   if (MODE == kScanLocal && blockIdx.z == 0 && threadIdx.x == 0)
     a.chunk_decay[(int64_t)blockIdx.y * a.heads + h] = total_decay;
@@ -302,17 +333,19 @@ __global__ __launch_bounds__(kScanSlices* kScanCols) void ssm_combine_kernel(Sca
 
 template <int NI>
 static void launch_scan(const ScanArgs& a, int num_entries, int num_chunks, hipStream_t stream) {
-  const dim3 block(kScanSlices * kScanCols);
-  const unsigned z = (a.P + kScanCols - 1) / kScanCols;
+  const dim3 block(kScanThreads);
+  const unsigned z = (a.P + kScanBlockCols - 1) / kScanBlockCols;
+  const size_t lds = (size_t)(kScanStage * (2 * a.N + kScanBlockCols + 2)) * sizeof(float);
   if (num_chunks <= 0) {
-    hipLaunchKernelGGL((ssm_scan_kernel<NI, kScanWhole>), dim3(a.heads, num_entries, z), block, 0,
-                       stream, a);
+    hipLaunchKernelGGL((ssm_scan_kernel<NI, kScanWhole>), dim3(a.heads, num_entries, z), block,
+                       lds, stream, a);
     return;
   }
-  hipLaunchKernelGGL((ssm_scan_kernel<NI, kScanLocal>), dim3(a.heads, num_chunks, z), block, 0,
+  hipLaunchKernelGGL((ssm_scan_kernel<NI, kScanLocal>), dim3(a.heads, num_chunks, z), block, lds,
                      stream, a);
-  hipLaunchKernelGGL(ssm_combine_kernel<NI>, dim3(a.heads, num_entries, z), block, 0, stream, a);
-  hipLaunchKernelGGL((ssm_scan_kernel<NI, kScanOutput>), dim3(a.heads, num_chunks, z), block, 0,
+  hipLaunchKernelGGL(ssm_combine_kernel<NI>, dim3(a.heads, num_entries, (a.P + kScanCols - 1) / kScanCols),
+                     dim3(kScanSlices * kScanCols), 0, stream, a);
+  hipLaunchKernelGGL((ssm_scan_kernel<NI, kScanOutput>), dim3(a.heads, num_chunks, z), block, lds,
                      stream, a);
 }
 

@@ -85,6 +85,12 @@ class Dispatch:
     # as much as 130 walked tokens whatever its length.
     scan_whole_tokens: int = 128
 
+    # ---- latent attention on the matrix cores: a wavefront per tile of 16 (token, head)
+    # rows.  A step with fewer tiles than this shares each tile's keys out over wavefronts
+    # in runs of at least `latent_split_keys` keys, up to about this many wavefronts.
+    latent_full_tiles: int = 1024
+    latent_split_keys: int = 64
+
 
 #: what each table was measured on -> the table
 MEASURED: dict[str, Dispatch] = {

@@ -1151,9 +1151,57 @@ class HipOps:
         self._check_latent(cache, table, batch, dl)
         pos, eot, _, _ = self._batch_ptrs(batch, T)
         out = torch.empty(T, heads, kv_rank, dtype=out_dtype, device=self.device)
+        if cache.k_pages.dtype == torch.bfloat16 and self.latent_mfma and \
+                self.lib.ts_latent_attention_mfma_fits(kv_rank, rot_dim) == 1:
+            self._latent_attention_mfma(qa, out, batch, table, cache, heads, kv_rank, rot_dim,
+                                        scale, window)
+            return out
         self._call(self.lib.ts_latent_attention, _ptr(qa), _ptr(cache.k_pages),
                    _TYPE_CODE[cache.k_pages.dtype], _ptr(out), _TYPE_CODE[out_dtype], pos, eot,
                    _ptr(table),
                    table.shape[1], cache.page_size, T, heads, kv_rank, rot_dim,
                    int(window) if window else 0, c_float(scale), self._stream())
         return out
+
+    #: False sends bfloat16 pages to the float32 multiply-add kernel as well
+    latent_mfma = True
+
+    def _latent_attention_mfma(self, qa, out, batch, table, cache, heads, kv_rank, rot_dim,
+                               scale, window):
+        """The matrix-core kernel: tiles of 16 (token, head) rows of one entry, made on the
+        host once a step and head count; where they are few, each tile's keys are shared out
+        over several wavefronts and merged."""
+        d = self.dispatch
+        counts = [-(-n * heads // 16) for n in batch.q_lens]
+        # few tiles: one wavefront a workgroup, every tile's keys shared out; many: four
+        # tiles of one entry to a workgroup, which walk their keys together
+        waves = 1 if sum(counts) < d.latent_full_tiles else 4
+        key = ("latent_tiles", heads, waves)
+        if key not in batch.plans:
+            tiles, row = [], 0
+            for e, n in enumerate(batch.q_lens):
+                rows = n * heads
+                tiles += [(row + i, min(16, rows - i), e) for i in range(0, rows, 16)]
+                while len(tiles) % waves:
+                    tiles.append((row, 0, e))           # an empty tile fills the workgroup
+                row += rows
+            batch.plans[key] = (self._upload_ints(tiles), len(tiles))
+        tiles, num_tiles = batch.plans[key]
+        # the longest run of keys a workgroup can have: the window and its own tokens, or
+        # the longest context
+        span = batch.max_ctx_len if not window else min(batch.max_ctx_len, window + 16 * waves)
+        splits = 1
+        if waves == 1:
+            splits = max(1, min(-(-span // d.latent_split_keys), d.latent_full_tiles // num_tiles))
+        per = -(-(-(-span // splits) + 32) // 32) * 32 if splits > 1 else 1 << 30
+        part_o = part_ml = None
+        if splits > 1:
+            part_o = torch.empty(num_tiles, splits, 16, kv_rank, dtype=torch.float32,
+                                 device=self.device)
+            part_ml = torch.empty(num_tiles, splits, 16, 2, dtype=torch.float32,
+                                  device=self.device)
+        self._call(self.lib.ts_latent_attention_mfma, _ptr(qa), _ptr(cache.k_pages), _ptr(out),
+                   _TYPE_CODE[out.dtype], _ptr(tiles), num_tiles, waves, _ptr(batch.positions),
+                   _ptr(table), table.shape[1], cache.page_size, heads, kv_rank, rot_dim,
+                   int(window) if window else 0, c_float(scale), per, splits, _ptr(part_o),
+                   _ptr(part_ml), self._stream())
