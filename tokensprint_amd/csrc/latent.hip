@@ -269,8 +269,9 @@ struct LatentMfmaArgs {
 
 constexpr int kLatentPad = 8;     // elements between staged rows: operand reads spread over banks
 
-// The wavefronts of a workgroup (four where keys are not shared out, else one) take
-// consecutive tiles of one entry and walk the union of their keys together: each block of
+// The wavefronts of a workgroup take consecutive tiles of one entry (where keys are shared
+// out, one tile and three empty ones, which only help load) and walk the union of their
+// keys together: each block of
 // 32 cached rows is staged in LDS once by all of them (16-byte loads, rows that are not
 // there as zeros), and both operands come from there: the K operand as 16 bytes of a row,
 // the C^T operand as eight 2-byte reads of a column.  A tile with no rows only helps load.
@@ -333,6 +334,7 @@ __global__ __launch_bounds__(4 * kWave) void latent_attention_mfma_kernel(Latent
       if (part == 0) krow_s[key] = row;
     }
     __syncthreads();
+    if (__builtin_amdgcn_readfirstlane(nrows) <= 0) continue;   // an empty tile only loads
     f32x4_l st[2];
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk) {

@@ -175,6 +175,7 @@ constexpr int kScanThreads = 128;          // the walking kernel: 8 slices x 16 
 constexpr int kScanPerThread = 4;          // columns a thread owns
 constexpr int kScanBlockCols = kScanThreads / kScanSlices * kScanPerThread;   // 64
 constexpr int kScanStage = 16;             // tokens staged in LDS at a time
+static_assert(kScanStage * kScanBlockCols == 8 * kScanThreads, "a stage's x: eight loads a thread");
 
 // Thread (cg, s) = (tid / 8, tid % 8) keeps rows s, s + 8, ... of four columns in registers.
 // Sixteen tokens' operands (B, C, the workgroup's columns of x, the step and the decay,
@@ -225,14 +226,42 @@ __global__ __launch_bounds__(kScanThreads) void ssm_scan_kernel(ScanArgs a) {
   for (int t0 = first; t0 < end; t0 += kScanStage) {
     const int nt = min(kScanStage, end - t0);
     __syncthreads();                                  // the stage before has been walked
-    for (int i = threadIdx.x; i < nt * N; i += kScanThreads) {
-      const float* row = a.xbc + (int64_t)(t0 + i / N) * a.channels;
-      B_s[i] = row[b_col + i % N];
-      if (MODE != kScanLocal) C_s[i] = row[c_col + i % N];
-    }
-    for (int i = threadIdx.x; i < nt * kScanBlockCols; i += kScanThreads) {
-      const int tt = i / kScanBlockCols, c = i % kScanBlockCols;
-      x_s[i] = col0 + c < a.P ? a.xbc[(int64_t)(t0 + tt) * a.channels + h * a.P + col0 + c] : 0.f;
+    // Loads in batches of eight, all issued before the first is stored, so that a stage
+    // costs a few trips to memory and not one per element.
+    {
+      const int total = nt * N;
+      constexpr int U = 8;
+      for (int base = 0; base < total; base += kScanThreads * U) {
+        float vb[U], vc[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int i = base + u * kScanThreads + threadIdx.x;
+          vb[u] = vc[u] = 0.f;
+          if (i < total) {
+            const float* row = a.xbc + (int64_t)(t0 + i / N) * a.channels;
+            vb[u] = row[b_col + i % N];
+            if (MODE != kScanLocal) vc[u] = row[c_col + i % N];
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int i = base + u * kScanThreads + threadIdx.x;
+          if (i < total) {
+            B_s[i] = vb[u];
+            if (MODE != kScanLocal) C_s[i] = vc[u];
+          }
+        }
+      }
+      float vx[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {         // 16 tokens x 64 columns: eight a thread
+        const int i = u * kScanThreads + threadIdx.x;
+        const int tt = i / kScanBlockCols, c = i % kScanBlockCols;
+        vx[u] = (tt < nt && col0 + c < a.P)
+            ? a.xbc[(int64_t)(t0 + tt) * a.channels + h * a.P + col0 + c] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) x_s[u * kScanThreads + threadIdx.x] = vx[u];
     }
     if (threadIdx.x < nt) {
       const float d = softplus_f(a.proj[(int64_t)(t0 + threadIdx.x) * a.ld + a.dt_col + h] + bias);
@@ -311,16 +340,31 @@ __global__ __launch_bounds__(kScanSlices* kScanCols) void ssm_combine_kernel(Sca
     const int n = s + kScanSlices * i;
     S[i] = (!fresh && n < N) ? st[(int64_t)n * a.P + p] : 0.f;
   }
-  for (int c = a.entry_chunks[e]; c < a.entry_chunks[e + 1]; ++c) {
+  const int c_begin = a.entry_chunks[e], c_end = a.entry_chunks[e + 1];
+  float next[NI], next_decay = 0.f;
+  auto fetch = [&](int c) {                 // a chunk's contribution, ahead of its turn
+    const float* cs = a.chunk_state + ((int64_t)c * a.heads + h) * N * a.P;
+    next_decay = a.chunk_decay[(int64_t)c * a.heads + h];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int n = s + kScanSlices * i;
+      next[i] = n < N ? cs[(int64_t)n * a.P + p] : 0.f;
+    }
+  };
+  if (c_begin < c_end) fetch(c_begin);
+  for (int c = c_begin; c < c_end; ++c) {
     float* cs = a.chunk_state + ((int64_t)c * a.heads + h) * N * a.P;
-    const float decay = a.chunk_decay[(int64_t)c * a.heads + h];
+    float local[NI];
+    const float decay = next_decay;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) local[i] = next[i];
+    if (c + 1 < c_end) fetch(c + 1);
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
       const int n = s + kScanSlices * i;
       if (n < N) {
-        const float local = cs[(int64_t)n * a.P + p];
         cs[(int64_t)n * a.P + p] = S[i];
-        S[i] = fmaf(decay, S[i], local);
+        S[i] = fmaf(decay, S[i], local[i]);
       }
     }
   }

@@ -1173,17 +1173,20 @@ class HipOps:
         over several wavefronts and merged."""
         d = self.dispatch
         counts = [-(-n * heads // 16) for n in batch.q_lens]
-        # few tiles: one wavefront a workgroup, every tile's keys shared out; many: four
-        # tiles of one entry to a workgroup, which walk their keys together
+        # many tiles: four of one entry to a workgroup, which walk their keys together; few:
+        # one tile a workgroup (and three empty ones), every tile's keys shared out
         waves = 1 if sum(counts) < d.latent_full_tiles else 4
         key = ("latent_tiles", heads, waves)
         if key not in batch.plans:
             tiles, row = [], 0
             for e, n in enumerate(batch.q_lens):
                 rows = n * heads
-                tiles += [(row + i, min(16, rows - i), e) for i in range(0, rows, 16)]
-                while len(tiles) % waves:
-                    tiles.append((row, 0, e))           # an empty tile fills the workgroup
+                for i in range(0, rows, 16):
+                    tiles.append((row + i, min(16, rows - i), e))
+                    while waves == 1 and len(tiles) % 4:
+                        tiles.append((row, 0, e))       # empty tiles fill the workgroup
+                while len(tiles) % 4:
+                    tiles.append((row, 0, e))
                 row += rows
             batch.plans[key] = (self._upload_ints(tiles), len(tiles))
         tiles, num_tiles = batch.plans[key]
@@ -1192,7 +1195,8 @@ class HipOps:
         span = batch.max_ctx_len if not window else min(batch.max_ctx_len, window + 16 * waves)
         splits = 1
         if waves == 1:
-            splits = max(1, min(-(-span // d.latent_split_keys), d.latent_full_tiles // num_tiles))
+            splits = max(1, min(-(-span // d.latent_split_keys),
+                                d.latent_full_tiles // (num_tiles // 4)))
         per = -(-(-(-span // splits) + 32) // 32) * 32 if splits > 1 else 1 << 30
         part_o = part_ml = None
         if splits > 1:
@@ -1201,7 +1205,7 @@ class HipOps:
             part_ml = torch.empty(num_tiles, splits, 16, 2, dtype=torch.float32,
                                   device=self.device)
         self._call(self.lib.ts_latent_attention_mfma, _ptr(qa), _ptr(cache.k_pages), _ptr(out),
-                   _TYPE_CODE[out.dtype], _ptr(tiles), num_tiles, waves, _ptr(batch.positions),
+                   _TYPE_CODE[out.dtype], _ptr(tiles), num_tiles, 4, _ptr(batch.positions),
                    _ptr(table), table.shape[1], cache.page_size, heads, kv_rank, rot_dim,
                    int(window) if window else 0, c_float(scale), per, splits, _ptr(part_o),
                    _ptr(part_ml), self._stream())
