@@ -382,6 +382,27 @@ def op_times(model, page, entries_of, reps=3):
     return runs[len(runs) // 2]
 
 
+def zonopel_profile_step(args) -> int:
+    """Four eager steps of the Zonopel model of `--compare-size` (default 1b-layers): a
+    2,048-token prompt, or a decode step of eight requests at 2,048 tokens; for a profiler."""
+    import torch
+    from tokensprint_amd.engine.assemble import random_model
+    from tokensprint_amd.engine.runner import ModelRunner
+    zono, _ = compare_configs(COMPARE_SIZES[args.compare_size or "1b-layers"])
+    _, model = random_model(zono, 0, args.dtype, "cuda:0")
+    make = prefill_entries(2048) if args.profile_zonopel == "prefill" else decode_entries(8, 2048)
+    lengths = make(None)
+    runner = ModelRunner(model, page_size=16, num_pages=sum(-(-n // 16) + 1 for n in lengths),
+                         num_slots=len(lengths))
+    batch = runner.build(make(runner))
+    for _ in range(4):
+        batch.plans.clear()
+        runner.run(batch)
+    torch.cuda.synchronize()
+    print(json.dumps({"profiled": args.profile_zonopel, "steps": 4}))
+    return 0
+
+
 def zonopel_compare(args) -> int:
     """Prefill and decode throughput of Zonopel beside Qwen3 at equal sizes, and the time of
     every kind of kernel in a 2,048-token prompt and in a decode step of eight requests.
@@ -447,6 +468,9 @@ def main() -> int:
                     help="instead of the benchmark: Zonopel beside Qwen3 at equal sizes "
                          "(prefill, decode, time per kind of kernel); prints its own line")
     ap.add_argument("--compare-size", default=None, help="with --compare-zonopel: one size only")
+    ap.add_argument("--profile-zonopel", default=None, choices=["prefill", "decode"],
+                    help="instead of the benchmark: four eager steps of the Zonopel model of "
+                         "--compare-size, for a profiler")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -455,6 +479,8 @@ def main() -> int:
     import torch
     from tokensprint_amd.config import load_named_config
 
+    if args.profile_zonopel:
+        return zonopel_profile_step(args)
     if args.compare_zonopel:
         return zonopel_compare(args)
     raw = load_named_config(args.model)
