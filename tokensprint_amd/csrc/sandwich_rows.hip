@@ -16,6 +16,18 @@ __device__ __forceinline__ float inv_rms(float sumsq, int n, float eps) {
   return 1.0f / sqrtf(sumsq / (float)n + eps);
 }
 
+// A thread keeps the first kRowItems elements of its share of a row in registers between
+// the passes over the row (sum of squares, then the scaled values), so a row of up to
+// kRowItems x threads elements is read once; what lies beyond is read again.  A step of
+// few rows is a chain of trips to memory and barriers, and this halves the trips.
+constexpr int kRowItems = 8;
+
+// Threads for a row of `width` elements: eight elements a thread, 64 to 1024 threads.
+static int row_threads(int width) {
+  int t = ((width + kRowItems - 1) / kRowItems + 63) / 64 * 64;
+  return t < 64 ? 64 : (t > 1024 ? 1024 : t);
+}
+
 // ---------------------------------------------------------------- bigram embedding
 template <typename TW>
 __global__ __launch_bounds__(256) void bigram_embed_kernel(
@@ -81,19 +93,37 @@ extern "C" int ts_bigram_embed(const void* table, const void* bigram, int table_
 // ---------------------------------------------------------------- add of a normalised output
 // resid += delta / rms(delta) * post_w; with NORM also out = resid / rms(resid) * norm_w.
 template <typename TO, bool NORM>
-__global__ __launch_bounds__(256) void postnorm_add_kernel(
+__global__ __launch_bounds__(1024) void postnorm_add_kernel(
     float* __restrict__ resid, const float* __restrict__ delta, const float* __restrict__ post_w,
     const float* __restrict__ norm_w, TO* __restrict__ out, int width, float post_eps,
     float norm_eps) {
   __shared__ float scratch[16];
   const int64_t row = blockIdx.x;
+  const int nt = blockDim.x;
   float* x = resid + row * width;
   const float* d = delta + row * width;
+  float dc[kRowItems], xc[kRowItems];
   float ss = 0.f;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) ss += d[i] * d[i];
+#pragma unroll
+  for (int k = 0; k < kRowItems; ++k) {
+    const int i = threadIdx.x + k * nt;
+    dc[k] = i < width ? d[i] : 0.f;
+    xc[k] = i < width ? x[i] : 0.f;
+    ss += dc[k] * dc[k];
+  }
+  for (int i = threadIdx.x + kRowItems * nt; i < width; i += nt) ss += d[i] * d[i];
   const float r = inv_rms(block_sum(ss, scratch), width, post_eps);
   float ss2 = 0.f;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+#pragma unroll
+  for (int k = 0; k < kRowItems; ++k) {
+    const int i = threadIdx.x + k * nt;
+    if (i < width) {
+      xc[k] = xc[k] + dc[k] * r * post_w[i];
+      x[i] = xc[k];
+      ss2 += xc[k] * xc[k];
+    }
+  }
+  for (int i = threadIdx.x + kRowItems * nt; i < width; i += nt) {
     const float v = x[i] + d[i] * r * post_w[i];
     x[i] = v;
     ss2 += v * v;
@@ -101,8 +131,14 @@ __global__ __launch_bounds__(256) void postnorm_add_kernel(
   if (NORM) {
     const float r2 = inv_rms(block_sum(ss2, scratch), width, norm_eps);
     TO* o = out + row * width;
+#pragma unroll
+    for (int k = 0; k < kRowItems; ++k) {
+      const int i = threadIdx.x + k * nt;
+      if (i < width) o[i] = from_f32<TO>(xc[k] * r2 * norm_w[i]);
+    }
     // each thread reads back the elements it wrote itself
-    for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = from_f32<TO>(x[i] * r2 * norm_w[i]);
+    for (int i = threadIdx.x + kRowItems * nt; i < width; i += nt)
+      o[i] = from_f32<TO>(x[i] * r2 * norm_w[i]);
   }
 }
 
@@ -112,13 +148,13 @@ extern "C" int ts_postnorm_add(float* resid, const float* delta, const float* po
   if (rows <= 0) return 0;
   if (width <= 0) TS_FAIL("postnorm_add: bad width %d", width);
   if (norm_w == nullptr) {
-    hipLaunchKernelGGL((postnorm_add_kernel<float, false>), dim3(rows), dim3(256), 0, stream,
-                       resid, delta, post_w, nullptr, nullptr, width, post_eps, 0.f);
+    hipLaunchKernelGGL((postnorm_add_kernel<float, false>), dim3(rows), dim3(row_threads(width)),
+                       0, stream, resid, delta, post_w, nullptr, nullptr, width, post_eps, 0.f);
   } else {
     TS_DISPATCH_TYPE(out_type, TO,
-                     hipLaunchKernelGGL((postnorm_add_kernel<TO, true>), dim3(rows), dim3(256), 0,
-                                        stream, resid, delta, post_w, norm_w, (TO*)out, width,
-                                        post_eps, norm_eps));
+                     hipLaunchKernelGGL((postnorm_add_kernel<TO, true>), dim3(rows),
+                                        dim3(row_threads(width)), 0, stream, resid, delta, post_w,
+                                        norm_w, (TO*)out, width, post_eps, norm_eps));
   }
   TS_CHECK_LAUNCH("postnorm_add");
   return 0;
@@ -129,42 +165,60 @@ extern "C" int ts_postnorm_add(float* resid, const float* delta, const float* po
 // h_(t-1) is recomputed from the row before inside a portion, read from the request's
 // state at a portion's first token, and zero at position 0.
 template <typename TO>
-__global__ __launch_bounds__(256) void norm_token_shift_kernel(
+__global__ __launch_bounds__(1024) void norm_token_shift_kernel(
     const float* __restrict__ resid, const float* __restrict__ norm_w,
     const float* __restrict__ shift_w, float* __restrict__ state, TO* __restrict__ out,
     const int* __restrict__ positions, const int* __restrict__ entry_of_token,
     const int* __restrict__ q_start, const int* __restrict__ slot_ids, int width, float eps) {
   __shared__ float scratch[16];
-  const int t = blockIdx.x;
+  const int t = blockIdx.x, nt = blockDim.x;
   const int e = entry_of_token[t];
   const int first = q_start[e], last = q_start[e + 1] - 1;
   const bool is_first = t == first;
   const bool from_state = is_first && positions[t] > 0;
+  const bool other_last = is_first && last != t;
   const float* x = resid + (int64_t)t * width;
   const float* xp = resid + (int64_t)(t - 1) * width;
   const float* xl = resid + (int64_t)last * width;
   float* st = state + (int64_t)slot_ids[e] * width;
-  float ss = 0.f, ssp = 0.f, ssl = 0.f;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) ss += x[i] * x[i];
-  const float r = inv_rms(block_sum(ss, scratch), width, eps);
-  float rp = 0.f, rl = r;
-  if (!is_first) {
-    for (int i = threadIdx.x; i < width; i += blockDim.x) ssp += xp[i] * xp[i];
-    rp = inv_rms(block_sum(ssp, scratch), width, eps);
-  } else if (last != t) {
-    for (int i = threadIdx.x; i < width; i += blockDim.x) ssl += xl[i] * xl[i];
-    rl = inv_rms(block_sum(ssl, scratch), width, eps);
+  // the row, and the one other row this workgroup needs (the row before, or the portion's
+  // last row whose norm goes into the state), both kept in registers
+  const float* y = !is_first ? xp : xl;
+  const bool need_y = !is_first || other_last;
+  float xc[kRowItems], yc[kRowItems];
+  float ss = 0.f, ssy = 0.f;
+#pragma unroll
+  for (int k = 0; k < kRowItems; ++k) {
+    const int i = threadIdx.x + k * nt;
+    xc[k] = i < width ? x[i] : 0.f;
+    yc[k] = (need_y && i < width) ? y[i] : 0.f;
+    ss += xc[k] * xc[k];
+    ssy += yc[k] * yc[k];
   }
+  for (int i = threadIdx.x + kRowItems * nt; i < width; i += nt) {
+    ss += x[i] * x[i];
+    if (need_y) ssy += y[i] * y[i];
+  }
+  const float r = inv_rms(block_sum(ss, scratch), width, eps);
+  float ry = r;
+  if (need_y) ry = inv_rms(block_sum(ssy, scratch), width, eps);
   TO* o = out + (int64_t)t * width;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+  auto finish = [&](int i, float xv, float yv) {
     const float w = norm_w[i];
-    const float h = x[i] * r * w;
+    const float h = xv * r * w;
     float prev = 0.f;
-    if (!is_first) prev = xp[i] * rp * w;
+    if (!is_first) prev = yv * ry * w;
     else if (from_state) prev = st[i];
     o[i] = from_f32<TO>(h + (prev - h) * shift_w[i]);
-    if (is_first) st[i] = xl[i] * rl * w;
+    if (is_first) st[i] = other_last ? yv * ry * w : h;
+  };
+#pragma unroll
+  for (int k = 0; k < kRowItems; ++k) {
+    const int i = threadIdx.x + k * nt;
+    if (i < width) finish(i, xc[k], yc[k]);
   }
+  for (int i = threadIdx.x + kRowItems * nt; i < width; i += nt)
+    finish(i, x[i], need_y ? y[i] : 0.f);
 }
 
 extern "C" int ts_norm_token_shift(const float* resid, const float* norm_w, float eps,
@@ -175,9 +229,10 @@ extern "C" int ts_norm_token_shift(const float* resid, const float* norm_w, floa
   if (num_tokens <= 0) return 0;
   if (width <= 0) TS_FAIL("norm_token_shift: bad width %d", width);
   TS_DISPATCH_TYPE(out_type, TO,
-                   hipLaunchKernelGGL(norm_token_shift_kernel<TO>, dim3(num_tokens), dim3(256), 0,
-                                      stream, resid, norm_w, shift_w, state, (TO*)out, positions,
-                                      entry_of_token, q_start, slot_ids, width, eps));
+                   hipLaunchKernelGGL(norm_token_shift_kernel<TO>, dim3(num_tokens),
+                                      dim3(row_threads(width)), 0, stream, resid, norm_w, shift_w,
+                                      state, (TO*)out, positions, entry_of_token, q_start,
+                                      slot_ids, width, eps));
   TS_CHECK_LAUNCH("norm_token_shift");
   return 0;
 }
@@ -185,29 +240,44 @@ extern "C" int ts_norm_token_shift(const float* resid, const float* norm_w, floa
 // ---------------------------------------------------------------- PolyNorm
 // out = a z/rms(z) + b z^2/rms(z^2) + c z^3/rms(z^3) + e, powers element by element.
 template <typename TO>
-__global__ __launch_bounds__(256) void polynorm_kernel(const float* __restrict__ z,
-                                                       const float* __restrict__ coef,
-                                                       TO* __restrict__ out, int width,
-                                                       float eps) {
+__global__ __launch_bounds__(1024) void polynorm_kernel(const float* __restrict__ z,
+                                                        const float* __restrict__ coef,
+                                                        TO* __restrict__ out, int width,
+                                                        float eps) {
   __shared__ float scratch[16];
   const int64_t row = blockIdx.x;
+  const int nt = blockDim.x;
   const float* x = z + row * width;
+  float zc[kRowItems];
   float s2 = 0.f, s4 = 0.f, s6 = 0.f;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const float v = x[i], v2 = v * v, v3 = v2 * v;
+  auto add = [&](float v) {
+    const float v2 = v * v, v3 = v2 * v;
     s2 += v2;
     s4 += v2 * v2;
     s6 += v3 * v3;
+  };
+#pragma unroll
+  for (int k = 0; k < kRowItems; ++k) {
+    const int i = threadIdx.x + k * nt;
+    zc[k] = i < width ? x[i] : 0.f;
+    add(zc[k]);
   }
+  for (int i = threadIdx.x + kRowItems * nt; i < width; i += nt) add(x[i]);
   const float r1 = inv_rms(block_sum(s2, scratch), width, eps);
   const float r2 = inv_rms(block_sum(s4, scratch), width, eps);
   const float r3 = inv_rms(block_sum(s6, scratch), width, eps);
   const float a = coef[0], b = coef[1], c = coef[2], e = coef[3];
   TO* o = out + row * width;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const float v = x[i], v2 = v * v;
-    o[i] = from_f32<TO>(a * (v * r1) + b * (v2 * r2) + c * (v2 * v * r3) + e);
+  auto value = [&](float v) {
+    const float v2 = v * v;
+    return a * (v * r1) + b * (v2 * r2) + c * (v2 * v * r3) + e;
+  };
+#pragma unroll
+  for (int k = 0; k < kRowItems; ++k) {
+    const int i = threadIdx.x + k * nt;
+    if (i < width) o[i] = from_f32<TO>(value(zc[k]));
   }
+  for (int i = threadIdx.x + kRowItems * nt; i < width; i += nt) o[i] = from_f32<TO>(value(x[i]));
 }
 
 extern "C" int ts_polynorm(const float* z, const float* coef, void* out, int out_type, int rows,
@@ -215,8 +285,8 @@ extern "C" int ts_polynorm(const float* z, const float* coef, void* out, int out
   if (rows <= 0) return 0;
   if (width <= 0) TS_FAIL("polynorm: bad width %d", width);
   TS_DISPATCH_TYPE(out_type, TO,
-                   hipLaunchKernelGGL(polynorm_kernel<TO>, dim3(rows), dim3(256), 0, stream, z,
-                                      coef, (TO*)out, width, eps));
+                   hipLaunchKernelGGL(polynorm_kernel<TO>, dim3(rows), dim3(row_threads(width)), 0,
+                                      stream, z, coef, (TO*)out, width, eps));
   TS_CHECK_LAUNCH("polynorm");
   return 0;
 }
