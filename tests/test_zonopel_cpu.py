@@ -139,3 +139,40 @@ def test_random_weights_fit_the_declarations(tmp_path):
     assert decls["l4.mix.in"].shape == (2 * 24 + 2 * 9 + 2, 40) and "l4.mlp.up" not in decls
     d = write_random_model(tmp_path / "m", ZONO_A, 3, torch.bfloat16)
     load_model(d, "bfloat16", "cpu", ops=TorchOps())
+
+
+# ------------------------------------------------------------------ unusual layer lists
+
+
+def _run_drives(cfg, seed, page, tmp_path):
+    d = write_random_model(tmp_path / "m", cfg, seed, torch.float32, std=0.2)
+    pcfg, w = plain.read_model_dir(d)
+    _, model = load_model(d, "float32", "cpu", ops=TorchOps())
+    requests = {f"r{i}": random_prompt(n, cfg["vocab"], 300 + i) for i, n in enumerate([9, 30, 1, 18])}
+    ref = {rid: plain_logits(pcfg, w, t) for rid, t in requests.items()}
+    drives.compare(drives.drive_portions(runner_for(model, page, 10), requests), ref, *TOL)
+    drives.compare(drives.drive_mixed(runner_for(model, page, 10), requests), ref, *TOL)
+
+
+def test_only_recurrent_layers_and_weights_borrowed_from_a_later_layer(tmp_path):
+    """No layer keeps pages (the cache manager has no group at all); the first layer runs
+    with the second one's weights."""
+    from helpers import zonopel_config, zonopel_mamba
+    cfg = zonopel_config(width=24, vocab=50, eps=1e-5, scale=1.5, buckets=11, mul_prev=5,
+                         mul_cur=2, layers=[
+                             zonopel_mamba(heads=0, vdim=0, state=0, groups=0, conv=0,
+                                           norm_groups=0, weights_of=1),
+                             zonopel_mamba(heads=3, vdim=8, state=6, groups=3, conv=3,
+                                           norm_groups=3, ff=32)])
+    _run_drives(cfg, 21, 8, tmp_path)
+
+
+def test_only_attention_layers(tmp_path):
+    from helpers import zonopel_config, zonopel_latent
+    cfg = zonopel_config(width=24, vocab=50, eps=1e-5, scale=1.5, buckets=11, mul_prev=5,
+                         mul_cur=2, layers=[
+                             zonopel_latent(heads=2, dim=6, rot_dim=4, vdim=5, q_rank=10,
+                                            kv_rank=12, window=7, ff=None),
+                             zonopel_latent(heads=2, dim=6, rot_dim=4, vdim=5, q_rank=10,
+                                            kv_rank=12, window=7, ff=20)])
+    _run_drives(cfg, 22, 8, tmp_path)
