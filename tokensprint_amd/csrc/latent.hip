@@ -422,27 +422,44 @@ __global__ __launch_bounds__(4 * kWave) void latent_attention_mfma_kernel(Latent
 }
 
 // One workgroup per (tile, row): the shares' results weighted by exp(m_s - max m) and
-// divided by the summed weights of their l, shares in index order.
+// divided by the summed weights of their l, shares in index order.  The first wavefront
+// turns the shares' statistics into weights (in LDS); then every thread adds its columns
+// over the shares, eight loads at a time.
 template <typename TO>
 __global__ __launch_bounds__(128) void latent_attention_merge_kernel(LatentMfmaArgs a) {
+  extern __shared__ float w_s[];            // [splits] weights, then the reciprocal of their sum
   const int tile = blockIdx.x, r = blockIdx.y;
   if (r >= a.tiles[3 * tile + 1]) return;
   const int64_t base = (int64_t)tile * a.splits * 16 + r;
-  float mx = -INFINITY;
-  for (int s = 0; s < a.splits; ++s) mx = fmaxf(mx, a.part_ml[2 * (base + 16 * s)]);
-  float total = 0.f;
-  for (int s = 0; s < a.splits; ++s) {
-    const float ms = a.part_ml[2 * (base + 16 * s)];
-    if (ms != -INFINITY) total += a.part_ml[2 * (base + 16 * s) + 1] * expf(ms - mx);
+  if (threadIdx.x < kWave) {
+    float mx = -INFINITY;
+    for (int s = threadIdx.x; s < a.splits; s += kWave)
+      mx = fmaxf(mx, a.part_ml[2 * (base + 16 * s)]);
+    mx = wave_max(mx);
+    float total = 0.f;
+    for (int s = threadIdx.x; s < a.splits; s += kWave) {
+      const float ms = a.part_ml[2 * (base + 16 * s)];
+      const float w = ms == -INFINITY ? 0.f : expf(ms - mx);
+      w_s[s] = w;
+      total += a.part_ml[2 * (base + 16 * s) + 1] * w;
+    }
+    total = wave_sum(total);
+    if (threadIdx.x == 0) w_s[a.splits] = total > 0.f ? 1.0f / total : 0.f;
   }
-  const float inv = total > 0.f ? 1.0f / total : 0.f;
+  __syncthreads();
+  const float inv = w_s[a.splits];
   TO* orow = (TO*)a.out + (int64_t)(a.tiles[3 * tile] + r) * a.kv_rank;
   for (int d = threadIdx.x; d < a.kv_rank; d += blockDim.x) {
     float acc = 0.f;
-    for (int s = 0; s < a.splits; ++s) {
-      const float ms = a.part_ml[2 * (base + 16 * s)];
-      if (ms != -INFINITY) acc = fmaf(a.part_o[(base + 16 * s) * a.kv_rank + d], expf(ms - mx), acc);
+    int s = 0;
+    for (; s + 8 <= a.splits; s += 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = a.part_o[(base + 16 * (s + u)) * a.kv_rank + d];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) acc = fmaf(v[u], w_s[s + u], acc);
     }
+    for (; s < a.splits; ++s) acc = fmaf(a.part_o[(base + 16 * s) * a.kv_rank + d], w_s[s], acc);
     orow[d] = from_f32<TO>(acc * inv);
   }
 }
@@ -456,8 +473,8 @@ static int launch_latent_mfma(const LatentMfmaArgs& a, int num_tiles, int waves,
     hipLaunchKernelGGL((latent_attention_mfma_kernel<KS, DB, TO>),
                        dim3(num_tiles / waves, a.splits), dim3(waves * kWave), lds, stream, a);
     if (a.splits > 1)
-      hipLaunchKernelGGL(latent_attention_merge_kernel<TO>, dim3(num_tiles, 16), dim3(128), 0,
-                         stream, a);
+      hipLaunchKernelGGL(latent_attention_merge_kernel<TO>, dim3(num_tiles, 16), dim3(128),
+                         (size_t)(a.splits + 1) * sizeof(float), stream, a);
   });
   return 0;
 }

@@ -86,10 +86,13 @@ class Dispatch:
     scan_whole_tokens: int = 128
 
     # ---- latent attention on the matrix cores: a wavefront per tile of 16 (token, head)
-    # rows.  A step with fewer tiles than this shares each tile's keys out over wavefronts
-    # in runs of at least `latent_split_keys` keys, up to about this many wavefronts.
+    # rows.  A step with fewer tiles than this shares each tile's keys out over workgroups
+    # in runs of at least `latent_split_keys` keys (a multiple of 32), up to about this many
+    # workgroups.  A workgroup's time is its start (tile, positions, block table, queries:
+    # a chain of dependent loads) and then 10 to 15 us a block of 32 keys, so short runs win:
+    # 8 requests with 1,024 visible keys, 16 heads, rank 512: 78 us in runs of 96.
     latent_full_tiles: int = 1024
-    latent_split_keys: int = 64
+    latent_split_keys: int = 32
 
 
 #: what each table was measured on -> the table

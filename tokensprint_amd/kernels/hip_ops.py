@@ -1193,11 +1193,15 @@ class HipOps:
         # the longest run of keys a workgroup can have: the window and its own tokens, or
         # the longest context
         span = batch.max_ctx_len if not window else min(batch.max_ctx_len, window + 16 * waves)
-        splits = 1
+        # shares start at an absolute multiple of 32 at or below the first visible key, so
+        # up to 31 keys more than the span have to be covered
+        splits, per = 1, 1 << 30
         if waves == 1:
-            splits = max(1, min(-(-span // d.latent_split_keys),
-                                d.latent_full_tiles // (num_tiles // 4)))
-        per = -(-(-(-span // splits) + 32) // 32) * 32 if splits > 1 else 1 << 30
+            most = max(1, d.latent_full_tiles // (num_tiles // 4))
+            per = -(-max(d.latent_split_keys, -(-(span + 31) // most)) // 32) * 32
+            splits = -(-(span + 31) // per)
+            if splits == 1:
+                per = 1 << 30
         part_o = part_ml = None
         if splits > 1:
             part_o = torch.empty(num_tiles, splits, 16, kv_rank, dtype=torch.float32,
