@@ -177,12 +177,15 @@ constexpr int kScanBlockCols = kScanThreads / kScanSlices * kScanPerThread;   //
 constexpr int kScanStage = 16;             // tokens staged in LDS at a time
 static_assert(kScanStage * kScanBlockCols == 8 * kScanThreads, "a stage's x: eight loads a thread");
 
+// (The output pass is held to 168 registers so that three wavefronts share a SIMD: its
+// time went from 292 to 220 us at 64 heads of 64 columns and 128 state rows, 2,048 tokens.)
 // Thread (cg, s) = (tid / 8, tid % 8) keeps rows s, s + 8, ... of four columns in registers.
 // Sixteen tokens' operands (B, C, the workgroup's columns of x, the step and the decay,
 // computed once a token) are staged in LDS by all threads together, then walked in order:
 // a token costs a thread 2 NI + 3 LDS reads for 8 NI multiply-adds.
 template <int NI, int MODE>
-__global__ __launch_bounds__(kScanThreads) void ssm_scan_kernel(ScanArgs a) {
+__global__ __launch_bounds__(kScanThreads, (MODE == kScanOutput && NI <= 16) ? 3 : 1)
+void ssm_scan_kernel(ScanArgs a) {
   extern __shared__ float lds[];
   const int N = a.N;
   float* B_s = lds;                                  // [stage][N]
