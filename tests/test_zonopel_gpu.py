@@ -221,7 +221,8 @@ def test_recurrence_remembers_a_far_token(gpu_device):
 @pytest.mark.parametrize("cache_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads, dim, rot_dim, rot_dims, vdim, q_rank, kv_rank, window",
                          [(3, 8, 6, 4, 10, 12, 14, 5), (5, 16, 8, 8, 12, 24, 32, None),
-                          (4, 32, 16, 16, 32, 96, 64, 24), (16, 128, 64, 64, 128, 256, 512, 33)])
+                          (4, 32, 16, 16, 32, 96, 64, 24), (16, 128, 64, 64, 128, 256, 512, 33),
+                          (2, 16, 24, 24, 16, 32, 712, 9)])
 def test_latent_attention_kernels(gpu_device, cache_dtype, heads, dim, rot_dim, rot_dims, vdim,
                                   q_rank, kv_rank, window):
     ops = load_hip_ops(gpu_device)

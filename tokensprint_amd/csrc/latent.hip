@@ -131,9 +131,9 @@ extern "C" int ts_rotate_interleaved(void* x, int type, const int* positions, co
 // and with it the rounding depends only on the token's position and the window.  In a
 // tile, lane j scores key j (a dot product over the whole row); then the lanes turn to the
 // columns of c and add the tile's weighted rows, key by key in order.
-constexpr int kMaxLatent = 1024;              // kv_rank + rot_dim
+constexpr int kMaxLatent = 2048;              // kv_rank + rot_dim
 constexpr int kLatentWaves = 4;
-constexpr int kMaxRankPerLane = 8;            // kv_rank <= 512
+constexpr int kMaxRankPerLane = 16;           // kv_rank <= 1024
 
 template <typename TC, typename TO>
 __global__ __launch_bounds__(kLatentWaves* kWave) void latent_attention_kernel(
