@@ -176,3 +176,15 @@ def test_only_attention_layers(tmp_path):
                              zonopel_latent(heads=2, dim=6, rot_dim=4, vdim=5, q_rank=10,
                                             kv_rank=12, window=7, ff=20)])
     _run_drives(cfg, 22, 8, tmp_path)
+
+
+def test_the_architecture_is_registered_beside_the_others():
+    from model_registry import listing
+    from tokensprint_amd.config import architecture_names
+    assert {"Qwen3ForCausalLM", "Zonopel"} <= set(architecture_names())
+    assert "Zonopel" in listing()
+    # config.json names it with a single 'architecture' string
+    from tokensprint_amd.config.model_config import architecture_of
+    assert architecture_of(ZONO_B) == "Zonopel"
+    with pytest.raises(ConfigError, match="architecture"):
+        architecture_of({"width": 8})
