@@ -56,3 +56,20 @@ def test_a_request_that_leaves_early_is_an_error(model, tmp_path):
     with pytest.raises(RuntimeError, match="live before"):
         # room for fewer tokens than the prompts' skew and the steps need
         bench.decode_run(engine, 64, 512, 20, 5, 256, max_tokens=30)
+
+
+def test_compared_designs_are_of_equal_size():
+    """`bench.py --compare-zonopel` builds a Zonopel and a Qwen3 configuration per size with
+    the same width, depth, vocabulary and (within 2 %) number of parameters."""
+    import math
+
+    import bench
+    from tokensprint_amd.weights.random_init import declared_tensors
+    for name, size in bench.COMPARE_SIZES.items():
+        zono, qwen = bench.compare_configs(size)
+        count = [sum(math.prod(d.shape) for d in declared_tensors(raw).values())
+                 for raw in (zono, qwen)]
+        assert abs(count[0] - count[1]) <= 0.02 * count[0], (name, count)
+        assert zono["width"] == qwen["hidden_size"] and zono["vocab"] == qwen["vocab_size"]
+        assert len(zono["layers"]) == qwen["num_hidden_layers"]
+        assert {e["type"] for e in zono["layers"]} == {"mamba2", "latent_attention"}
