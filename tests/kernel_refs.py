@@ -194,6 +194,107 @@ class TorchOps:
         return (a * self._unit(z, eps) + b * self._unit(z2, eps) + c * self._unit(z2 * z, eps)
                 + e).to(out_dtype)
 
+    # ---------------------------------------------------------------- stream sums
+    def stream_add(self, resid, a, b, row):
+        if a is not None:
+            resid.add_(a.float() + b.float() if b is not None else a.float())
+        if row is not None:
+            resid.add_(row.float())
+
+    def scaled_sum(self, a, scale_a, b, scale_b):
+        return scale_a * a.float() + scale_b * b.float()
+
+    def take_columns(self, x, col, count, out_dtype):
+        return x[:, col:col + count].to(out_dtype).contiguous()
+
+    # ---------------------------------------------------------------- matrix-state mixers
+    def delta_gates(self, qkv, proj, beta_col, z, z_col, a_log, dt_bias, *, heads, kv_heads, dim,
+                    per_channel):
+        T = qkv.shape[0]
+        qk = kv_heads * dim
+        for c0, scale in ((0, dim ** -0.5), (qk, 1.0)):
+            x = qkv[:, c0:c0 + qk].view(T, kv_heads, dim)
+            x.mul_(torch.rsqrt(x.pow(2).sum(-1, keepdim=True) + 1e-6) * scale)
+        beta = torch.sigmoid(proj[:, beta_col:beta_col + heads].float())
+        n = heads * dim if per_channel else heads
+        pre = z[:, z_col:z_col + n].float() + dt_bias.float()
+        sp = torch.nn.functional.softplus(pre, threshold=30.0)
+        rate = torch.exp(a_log.float())
+        if per_channel:
+            g = torch.exp(-(rate[:, None] * sp.view(T, heads, dim))).view(T, n)
+        else:
+            g = torch.exp(-rate * sp)
+        return torch.cat([beta, g], dim=1).contiguous()
+
+    def linear_recurrence(self, x, q_col, k_col, v_col, batch, state, *, heads, kv_heads, dim,
+                          vdim, silu_inputs, decay=None, gates=None, per_channel=False,
+                          delta=False):
+        T = x.shape[0]
+        rep = heads // kv_heads
+
+        def part(col, n, size):
+            v = x[:, col:col + n * size].float()
+            if silu_inputs:
+                v = v * torch.sigmoid(v)
+            return v.view(T, n, size)
+
+        q = part(q_col, kv_heads, dim).repeat_interleave(rep, dim=1)
+        k = part(k_col, kv_heads, dim).repeat_interleave(rep, dim=1)
+        v = part(v_col, heads, vdim)
+        out = torch.empty(T, heads, vdim, dtype=torch.float32, device=x.device)
+        for b, lo, hi, slot, start in self._entries(batch):
+            S = state[slot].clone() if start > 0 else torch.zeros_like(state[slot])
+            for t in range(lo, hi):
+                if gates is None:
+                    S = S * decay.float()[:, None, None]
+                elif per_channel:
+                    S = S * gates[t, heads:].view(heads, dim, 1)
+                else:
+                    S = S * gates[t, heads:].view(heads, 1, 1)
+                if delta:
+                    pred = (S * k[t][:, :, None]).sum(1)
+                    u = gates[t, :heads, None] * (v[t] - pred)
+                else:
+                    u = v[t]
+                S = S + k[t][:, :, None] * u[:, None, :]
+                out[t] = (S * q[t][:, :, None]).sum(1)
+            state[slot] = S
+        return out.view(T, heads * vdim)
+
+    def norm_gate(self, y, gate_rows, gate_col, norm_w, *, groups, gate, eps, out_dtype):
+        T, inner = y.shape
+        width = inner // groups
+        yf = y.float().view(T, groups, width)
+        yf = yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps)
+        w = norm_w.float()
+        yf = yf * (w.view(1, 1, width) if w.numel() == width else w.view(1, groups, width))
+        z = gate_rows[:, gate_col:gate_col + inner].float()
+        act = torch.sigmoid(z) if gate == "sigmoid" else z * torch.sigmoid(z)
+        return (yf.view(T, inner) * act).to(out_dtype)
+
+    # ---------------------------------------------------------------- routed experts
+    def route_experts(self, logits, *, top, group_count, group_keep):
+        T, E = logits.shape
+        scores = torch.softmax(logits.float(), dim=-1)
+        per = E // group_count
+        best = scores.view(T, group_count, per).max(-1).values
+        kept = torch.zeros(T, group_count, dtype=torch.bool, device=logits.device)
+        kept.scatter_(1, best.topk(group_keep, dim=-1).indices, True)
+        allowed = kept[:, :, None].expand(T, group_count, per).reshape(T, E)
+        chosen = torch.where(allowed, scores, torch.full_like(scores, -1.0)).topk(top, -1).indices
+        picked = torch.gather(scores, 1, chosen)
+        out = torch.zeros_like(scores)
+        out.scatter_(1, chosen, picked / (picked.sum(-1, keepdim=True) + 1e-20))
+        return out
+
+    def expert_activation(self, gate_up, weights, inner, limit, out_dtype):
+        T, E = weights.shape
+        gu = gate_up.float().view(T, E, 2, inner)
+        g = torch.clamp(gu[:, :, 0], max=limit)
+        u = torch.clamp(gu[:, :, 1], -limit, limit)
+        y = g * torch.sigmoid(1.702 * g) * (u + 1.0) * weights.float()[:, :, None]
+        return y.view(T, E * inner).to(out_dtype)
+
     # ---------------------------------------------------------------- state-space mixer
     def conv_silu(self, proj, col, channels, weight, bias, batch, state):
         taps = weight.shape[1]
@@ -203,7 +304,8 @@ class TorchOps:
             hist = state[slot] if start > 0 else torch.zeros_like(state[slot])
             full = torch.cat([hist, u[lo:hi]], dim=0)           # [taps-1 + n, C]
             n = hi - lo
-            acc = bias.float().expand(n, channels).clone()
+            acc = bias.float().expand(n, channels).clone() if bias is not None \
+                else torch.zeros(n, channels, dtype=torch.float32, device=u.device)
             for k in range(taps):
                 acc = acc + full[k:k + n] * weight[:, k].float()
             out[lo:hi] = acc * torch.sigmoid(acc)

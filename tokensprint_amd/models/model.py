@@ -42,6 +42,7 @@ class Model:
         self.final_norm = build_part(NORMS, spec.final_norm, ctx)
         self.head = build_part(HEADS, spec.head, ctx)
         self.order = spec.order
+        self.enter_tables: dict[str, torch.Tensor] = {}
 
     # ------------------------------------------------------------ weights
     def parts(self):
@@ -53,7 +54,9 @@ class Model:
         return out
 
     def tensor_decls(self) -> dict[str, TensorDecl]:
-        decls: dict[str, TensorDecl] = {}
+        decls: dict[str, TensorDecl] = {
+            name: TensorDecl((rows, self.spec.width), role="vector", init=(-0.3, 0.3))
+            for name, rows in self.spec.enter_tables.items()}
         for part in self.parts():
             for name, decl in part.tensors().items():
                 if name in decls and (decls[name].shape != decl.shape
@@ -68,6 +71,7 @@ class Model:
     def load_tensors(self, tensors: dict[str, torch.Tensor]) -> None:
         for part in self.parts():
             part.load(tensors.get)
+        self.enter_tables = {name: tensors[name] for name in self.spec.enter_tables}
 
     # ------------------------------------------------------------ caches
     def cache_needs(self):
@@ -95,7 +99,11 @@ class Model:
             # what reads the stream after this run: the next run's block (the final norm
             # and the head take a plain delta)
             next_hint = self.blocks[self.order[r + 1].layer].entry_hint() \
-                if r + 1 < len(self.order) else None
+                if r + 1 < len(self.order) and self.order[r + 1].enter is None else None
+            if run.enter is not None:
+                # what is still to be added, then the row of this pass
+                ops.stream_add(resid, delta, None, self.enter_tables[run.enter[0]][run.enter[1]])
+                delta = None
             resid, delta = self.blocks[run.layer].forward(
                 resid, delta, batch, caches[owner], write_cache=run.cache_of is None,
                 next_hint=next_hint)
@@ -114,7 +122,8 @@ class Model:
         the embedding share one table): the weight traffic of a decode step."""
         seen, total = set(), 0
         for part in self.parts():
-            for t in part.step_read_tensors():
+            for t in part.step_read_tensors() + (
+                    list(self.enter_tables.values()) if part is self.final_norm else []):
                 if t.data_ptr() not in seen:
                     seen.add(t.data_ptr())
                     total += t.numel() * t.element_size()

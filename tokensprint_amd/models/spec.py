@@ -65,10 +65,14 @@ class Run:
 
     `cache_of` names the run (index into `ModelSpec.order`) whose cache this run
     uses; None means its own.  A run that uses another run's cache only reads it.
+    `enter` names a row of a [rows, width] tensor, (tensor name, row), that is added to the
+    residual stream right before this run (a pass of a repeated stretch of layers that
+    tells the layers which pass it is); None: nothing is added.
     """
 
     layer: int
     cache_of: int | None = None
+    enter: tuple[str, int] | None = None
 
 
 @dataclass(frozen=True)
@@ -84,6 +88,8 @@ class ModelSpec:
     head: PartSpec
     max_position: int
     eos_token_id: int | None = None       # the checkpoint's end-of-sequence token, if it names one
+    #: rows of every tensor a run's `enter` names: tensor name -> number of rows
+    enter_tables: Mapping[str, int] = field(default_factory=dict)
 
     def validate(self) -> None:
         if not self.order:
@@ -98,3 +104,8 @@ class ModelSpec:
                 if self.order[run.cache_of].cache_of is not None:
                     raise ValueError(
                         f"run {r} reads the cache of run {run.cache_of}, which owns none")
+            if run.enter is not None:
+                name, row = run.enter
+                if not 0 <= row < self.enter_tables.get(name, 0):
+                    raise ValueError(f"run {r} enters with row {row} of '{name}', which has "
+                                     f"{self.enter_tables.get(name, 0)} rows")

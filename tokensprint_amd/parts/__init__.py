@@ -1,5 +1,5 @@
 from tokensprint_amd.parts import (attention, block, feed_forward, latent_attention, mamba2,  # noqa: F401
-                                   norm, position)
+                                   norm, position, recurrent)
 from tokensprint_amd.parts.base import (
     BLOCKS, EMBEDDINGS, FEED_FORWARDS, FILTERS, HEADS, MIXERS, NORMS, POSITIONS, Block,
     BuildContext, FeedForward, Mixer, Norm, OutputHead, PagedKVNeed, PagedLatentNeed, Part,

@@ -117,3 +117,62 @@ class GroupedQueryAttention(StreamProducts, Mixer):
                                     num_kv_heads=self.nkv, head_dim=self.hd,
                                     scale=self.scale, window=self.window)
         return o.view(T, self.nq * self.hd)
+
+
+@register(MIXERS, "softmax_attention")
+class SoftmaxAttention(GroupedQueryAttention):
+    """Grouped-query softmax attention whose query/key size `dim`, value size `vdim`, score
+    scale and rotated dimensions are given one by one, with plain tensor names
+    ('<prefix>q', 'k', 'v', 'o').  The cache and the kernels know one head size: heads are
+    laid out in `head_dim` = the larger of the two sizes rounded up to 16, queries and keys
+    in the position encoding's layout with zeros in the places left over (they add nothing
+    to a score), values followed by zeros (their outputs meet zero columns of the output
+    projection).
+
+    params: prefix, heads, kv_heads, dim, vdim, scale, position (a 'rope_partial' encoding
+    of this head_dim, or None), window."""
+
+    def __init__(self, params, ctx):
+        p = dict(params)
+        self.dim, self.vdim = int(p["dim"]), int(p["vdim"])
+        p.update(num_heads=p["heads"], num_kv_heads=p["kv_heads"],
+                 head_dim=self.padded_head(self.dim, self.vdim), qk_norm=False)
+        super().__init__(p, ctx)
+        self.scale = float(p["scale"])
+        if self.position is not None and getattr(self.position, "head_dim", self.hd) != self.hd:
+            raise ValueError(f"{self.prefix}: the position encoding is laid out for heads of "
+                             f"{self.position.head_dim}, this mixer's are {self.hd}")
+
+    @staticmethod
+    def padded_head(dim: int, vdim: int) -> int:
+        return -(-max(dim, vdim) // 16) * 16
+
+    def tensors(self):
+        W, pre = self.ctx.width, self.prefix
+        return {pre + "q": TensorDecl((self.nq * self.dim, W)),
+                pre + "k": TensorDecl((self.nkv * self.dim, W)),
+                pre + "v": TensorDecl((self.nkv * self.vdim, W)),
+                pre + "o": TensorDecl((W, self.nq * self.vdim))}
+
+    def load(self, get):
+        pre, hd, W = self.prefix, self.hd, self.ctx.width
+        q, k, v, o = (get(pre + n) for n in "qkvo")
+        if len({q.dtype, k.dtype, v.dtype}) != 1:
+            raise ValueError(f"{pre}: q/k/v projection weights are stored in different dtypes")
+        layout = self.position.layout(self.dim) if self.position is not None \
+            else list(range(self.dim)) + [-1] * (hd - self.dim)
+        place = torch.tensor([j for j, src in enumerate(layout) if src >= 0], device=q.device)
+        src = torch.tensor([s for s in layout if s >= 0], device=q.device)
+
+        def heads_of(w, n, size, place, src):
+            out = torch.zeros(n, hd, W, dtype=w.dtype, device=w.device)
+            out[:, place] = w.view(n, size, W)[:, src]
+            return out.view(n * hd, W)
+
+        every = torch.arange(self.vdim, device=q.device)
+        self.w_qkv = torch.cat([heads_of(q, self.nq, self.dim, place, src),
+                                heads_of(k, self.nkv, self.dim, place, src),
+                                heads_of(v, self.nkv, self.vdim, every, every)], dim=0).contiguous()
+        w_o = torch.zeros(W, self.nq, hd, dtype=o.dtype, device=o.device)
+        w_o[:, :, :self.vdim] = o.view(W, self.nq, self.vdim)
+        self.w_o = w_o.view(W, self.nq * hd).contiguous()

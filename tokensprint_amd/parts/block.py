@@ -102,6 +102,24 @@ class SandwichNormBlock(Block):
         return resid, None
 
 
+@register(BLOCKS, "parallel_residual")
+class ParallelResidualBlock(Block):
+    """One norm whose output both sub-layers read: with h = norm(x),
+    x <- x + (mixer(h) + ffn(h)).  The feed-forward may be left out.  The stream leaves the
+    block summed up (no delta is handed on)."""
+
+    ROLES = {"mixer_norm": (NORMS, True), "mixer": (MIXERS, True),
+             "feed_forward": (FEED_FORWARDS, False)}
+
+    def forward(self, resid, delta, batch, cache, write_cache, next_hint=None):
+        h = self.mixer_norm.forward(resid) if delta is None \
+            else self.mixer_norm.add_forward(resid, delta)
+        mixed = self.mixer.forward(h, batch, cache, write_cache)
+        fed = self.feed_forward.forward(h, batch) if self.feed_forward is not None else None
+        self.ctx.ops.stream_add(resid, mixed, fed, None)
+        return resid, None
+
+
 @register(FILTERS, "token_shift")
 class TokenShift(StreamFilter):
     """h_t <- h_t + (h_(t-1) - h_t) * w, element by element, with h the norm of the stream

@@ -15,27 +15,28 @@ from tokensprint_amd.parts.base import FEED_FORWARDS, FeedForward, TensorDecl, r
 
 @register(FEED_FORWARDS, "swiglu")
 class SwiGLU(StreamProducts, FeedForward):
-    """params: prefix, inner_dim."""
+    """params: prefix, inner_dim, names (the tensors' names behind the prefix, gate, up and
+    down; default 'gate_proj.weight', 'up_proj.weight', 'down_proj.weight')."""
 
     def __init__(self, params, ctx):
         super().__init__(params, ctx)
         self.prefix = params["prefix"]
         self.inner = int(params["inner_dim"])
+        self.names = tuple(self.prefix + n for n in params.get(
+            "names", ("gate_proj.weight", "up_proj.weight", "down_proj.weight")))
         self.w_gate_up = self.w_down = None
 
     def tensors(self):
-        H, I, pre = self.ctx.width, self.inner, self.prefix
-        return {pre + "gate_proj.weight": TensorDecl((I, H)),
-                pre + "up_proj.weight": TensorDecl((I, H)),
-                pre + "down_proj.weight": TensorDecl((H, I))}
+        H, I = self.ctx.width, self.inner
+        gate, up, down = self.names
+        return {gate: TensorDecl((I, H)), up: TensorDecl((I, H)), down: TensorDecl((H, I))}
 
     def load(self, get):
-        pre = self.prefix
-        g, u = get(pre + "gate_proj.weight"), get(pre + "up_proj.weight")
+        g, u = get(self.names[0]), get(self.names[1])
         if g.dtype != u.dtype:
-            raise ValueError(f"{pre}: gate and up weights are stored in different dtypes")
+            raise ValueError(f"{self.prefix}: gate and up weights are stored in different dtypes")
         self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
-        self.w_down = get(pre + "down_proj.weight")
+        self.w_down = get(self.names[2])
 
     def stream_hint(self, norm):
         return self.first_product_hint(norm, self.w_gate_up, silu_mul=True)
@@ -82,3 +83,64 @@ class PolyNormMLP(FeedForward):
         z = self.ops.linear(h, self.w_up, torch.float32)
         act = self.ops.polynorm(z, self.coef, self.eps, self.ctx.dtype)
         return self.ops.linear(act, self.w_down, torch.float32)
+
+
+@register(FEED_FORWARDS, "routed_experts")
+class RoutedExperts(FeedForward):
+    """`experts` small gated feed-forwards of which a token uses `top`.
+
+    Router: scores = softmax over all experts of the float32 logits; experts stand in
+    `group_count` equal groups of neighbours, a group's score is its best expert's, and only
+    experts of the `group_keep` best groups can be chosen; of those the `top` with the
+    largest scores, weighed by their scores over the chosen scores' sum (+ 1e-20).
+    Expert: g = min(gate(h), limit), u = clamp(up(h), -limit, limit),
+    down(g sigmoid(1.702 g) (u + 1)).  The output is the weighted sum.
+
+    Every expert's gate and up rows are one product and every expert's down columns another:
+    the activation kernel writes a token's values times the expert's weight, and zeros for
+    the experts the token does not use, so the second product sums the chosen experts.
+
+    params: prefix, inner_dim (of one expert), experts, top, group_count, group_keep, limit."""
+
+    def __init__(self, params, ctx):
+        super().__init__(params, ctx)
+        p = params
+        self.prefix, self.inner = p["prefix"], int(p["inner_dim"])
+        self.experts, self.top = int(p["experts"]), int(p["top"])
+        self.group_count, self.group_keep = int(p["group_count"]), int(p["group_keep"])
+        self.limit = float(p["limit"])
+        if self.experts % self.group_count or self.group_keep > self.group_count or \
+                self.top > self.group_keep * (self.experts // self.group_count):
+            raise ValueError(f"{self.prefix}: {self.experts} experts in {self.group_count} groups, "
+                             f"{self.group_keep} kept, cannot give {self.top}")
+        self.w_router = self.w_gate_up = self.w_down = None
+
+    def tensors(self):
+        W, I, pre = self.ctx.width, self.inner, self.prefix
+        t = {pre + "router": TensorDecl((self.experts, W))}
+        for e in range(self.experts):
+            t[f"{pre}e{e}.gate"] = TensorDecl((I, W))
+            t[f"{pre}e{e}.up"] = TensorDecl((I, W))
+            t[f"{pre}e{e}.down"] = TensorDecl((W, I))
+        return t
+
+    def load(self, get):
+        pre = self.prefix
+        self.w_router = get(pre + "router")
+        rows, cols = [], []
+        for e in range(self.experts):
+            rows += [get(f"{pre}e{e}.gate"), get(f"{pre}e{e}.up")]
+            cols.append(get(f"{pre}e{e}.down"))
+        if len({r.dtype for r in rows + cols}) != 1:
+            raise ValueError(f"{pre}: expert weights are stored in different dtypes")
+        self.w_gate_up = torch.cat(rows, dim=0).contiguous()     # [E, gate | up] x width
+        self.w_down = torch.cat(cols, dim=1).contiguous()        # width x [E, inner]
+
+    def forward(self, h, batch):
+        ops = self.ops
+        logits = ops.linear(h, self.w_router, torch.float32)
+        weights = ops.route_experts(logits, top=self.top, group_count=self.group_count,
+                                    group_keep=self.group_keep)          # [T, experts]
+        gate_up = ops.linear(h, self.w_gate_up, self.ctx.dtype)
+        act = ops.expert_activation(gate_up, weights, self.inner, self.limit, self.ctx.dtype)
+        return ops.linear(act, self.w_down, torch.float32)

@@ -71,3 +71,55 @@ class InterleavedRotation(PositionEncoding):
         self.ops.rotate_interleaved_inplace(q, positions, self.freqs, self.dims, offset=0)
         if k is not None:
             self.ops.rotate_interleaved_inplace(k, positions, self.freqs, self.dims, offset=0)
+
+
+@register(POSITIONS, "rope_partial")
+class PartialRotaryEncoding(PositionEncoding):
+    """Rotate-half rotation of the first `dims` dimensions of a head of `head_dim`
+    dimensions: dimension i pairs with i + dims/2, angle position * base^(-2i/dims); the rest
+    passes unchanged.  The kernels rotate whole heads, pairing j with j + head_dim/2, so a
+    mixer that uses this lays its heads out by `layout()` (rotated first halves, the rest,
+    rotated second halves, the rest: a permutation of a head's dimensions, the same for
+    queries and keys, which changes no score) and the table holds cos = 1, sin = 0 for the
+    pairs that are not rotated.  Frequencies are rounded once from float64; angles and their
+    cosines and sines are float32, computed on the host.
+
+    params: dims, base, head_dim, max_position."""
+
+    def __init__(self, params, ctx):
+        super().__init__(params, ctx)
+        self.dims, self.base = int(params["dims"]), float(params["base"])
+        self.head_dim, self.max_position = int(params["head_dim"]), int(params["max_position"])
+        if self.dims % 2 or self.head_dim % 2 or not 2 <= self.dims <= self.head_dim:
+            raise ValueError(f"rotated dimensions ({self.dims}) must be even and fit the head "
+                             f"({self.head_dim}, even)")
+        half, r = self.head_dim // 2, self.dims // 2
+        i = torch.arange(r, dtype=torch.float64)
+        freqs = (self.base ** (-2.0 * i / self.dims)).to(torch.float32)
+        angles = torch.outer(torch.arange(self.max_position, dtype=torch.float32), freqs)
+        cos = torch.ones(self.max_position, half, dtype=torch.float32)
+        sin = torch.zeros(self.max_position, half, dtype=torch.float32)
+        cos[:, :r], sin[:, :r] = angles.cos(), angles.sin()
+        self.cos, self.sin = cos.contiguous().to(ctx.device), sin.contiguous().to(ctx.device)
+
+    def layout(self, dim: int) -> list[int]:
+        """For a head of `dim` given dimensions (dim <= head_dim): the given dimension that
+        stands at each of the `head_dim` places, -1 where a zero stands."""
+        half, r = self.head_dim // 2, self.dims // 2
+        rest = list(range(self.dims, dim))
+        first = list(range(r)) + rest[:half - r]
+        second = list(range(r, self.dims)) + rest[half - r:]
+        if len(second) > half:
+            raise ValueError(f"a head of {dim} dimensions does not fit {self.head_dim}")
+        return first + [-1] * (half - len(first)) + second + [-1] * (half - len(second))
+
+    def rotary_tables(self):
+        return self.cos, self.sin
+
+    def step_read_tensors(self):
+        return []
+
+    def apply(self, q, k, positions):
+        self.ops.rope_inplace(q, positions, self.cos, self.sin)
+        if k is not None:
+            self.ops.rope_inplace(k, positions, self.cos, self.sin)

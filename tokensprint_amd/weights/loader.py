@@ -110,8 +110,11 @@ def check_tensors(decls: dict[str, TensorDecl], source) -> None:
     have = set(source.names())
     missing = sorted(n for n, d in decls.items() if n not in have and not d.optional)
     unexpected = sorted(have - set(decls))
+    def fits(shape, declared):        # a declared size of -1 is read from the file
+        return len(shape) == len(declared) and all(
+            (d == -1 and s >= 1) or s == d for s, d in zip(shape, declared))
     wrong = sorted((n, decls[n].shape, source.shape(n)) for n in have & set(decls)
-                   if tuple(source.shape(n)) != tuple(decls[n].shape))
+                   if not fits(tuple(source.shape(n)), tuple(decls[n].shape)))
     if missing or unexpected or wrong:
         raise WeightsError(missing, unexpected, wrong)
 
@@ -128,7 +131,7 @@ def load_weights(model, source, run_dtype: torch.dtype, device, cast_32bit: bool
     decls = model.tensor_decls()
     check_tensors(decls, source)
     have = set(source.names())
-    needed = {n for part in model.parts() for n, d in part.tensors().items() if not d.optional}
+    needed = {n for n, d in decls.items() if not d.optional}
     tensors, kept_wide = {}, []
     for name in sorted(needed & have):
         t = source.read(name)

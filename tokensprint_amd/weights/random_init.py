@@ -45,6 +45,9 @@ def random_tensors(raw_config: dict, seed: int, dtype=torch.float32, std: float 
     for name, decl in sorted(declared_tensors(raw_config).items()):
         if decl.optional:
             continue
+        if any(d < 0 for d in decl.shape):
+            raise ValueError(f"{name}: a size that config.json leaves to the file "
+                             f"({decl.shape}); random weights need it in the configuration")
         gen = torch.Generator(device=device).manual_seed(_tensor_seed(seed, name))
         if decl.init is not None:
             lo, hi = decl.init
