@@ -1,0 +1,124 @@
+// Routed experts: the choice of a token's experts, and the experts' gated activation.
+#include "common.h"
+
+// ---------------------------------------------------------------- router
+// One wavefront per token.  scores = softmax(logits) over the E experts; the experts stand in
+// `group_count` equal groups of neighbours, a group's score is its best expert's, and only
+// the `group_keep` best groups' experts can be chosen; of those the `top` with the largest
+// scores (equal scores: the lower index).  weights[t][e] = score / (sum of the chosen scores
+// + 1e-20) for the chosen experts and 0 for the others.
+__global__ __launch_bounds__(256) void route_experts_kernel(
+    const float* __restrict__ logits, float* __restrict__ weights, int rows, int E, int top,
+    int group_count, int group_keep) {
+  extern __shared__ float lds[];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int64_t t = (int64_t)blockIdx.x * (blockDim.x / kWave) + wave;
+  const bool live = t < rows;                    // (every wavefront meets every barrier)
+  float* score = lds + (size_t)wave * (2 * E + group_count);
+  float* open = score + E;                       // the score while the expert can be chosen, else -1
+  float* best = open + E;                        // [group_count]
+  const float* z = logits + (live ? t : 0) * E;
+  float m = -INFINITY;
+  for (int e = lane; e < E; e += kWave) m = fmaxf(m, z[e]);
+  m = wave_max(m);
+  float sum = 0.f;
+  for (int e = lane; e < E; e += kWave) {
+    const float p = expf(z[e] - m);
+    score[e] = p;
+    sum += p;
+  }
+  sum = wave_sum(sum);
+  const float inv = 1.0f / sum;
+  const int per = E / group_count;
+  for (int e = lane; e < E; e += kWave) score[e] *= inv;
+  __syncthreads();
+  for (int g = lane; g < group_count; g += kWave) {
+    float b = -1.f;
+    for (int i = 0; i < per; ++i) b = fmaxf(b, score[g * per + i]);
+    best[g] = b;
+  }
+  __syncthreads();
+  for (int g = lane; g < group_count; g += kWave) {
+    int ahead = 0;                               // groups that come before this one
+    for (int o = 0; o < group_count; ++o)
+      ahead += best[o] > best[g] || (best[o] == best[g] && o < g);
+    const bool kept = ahead < group_keep;
+    for (int i = 0; i < per; ++i) open[g * per + i] = kept ? score[g * per + i] : -1.f;
+  }
+  __syncthreads();
+  float chosen_sum = 0.f;
+  float* w = weights + (live ? t : 0) * E;
+  for (int k = 0; k < top; ++k) {
+    float bv = -1.f;
+    int bi = E;
+    for (int e = lane; e < E; e += kWave)
+      if (open[e] > bv) bv = open[e], bi = e;    // ascending e: the lower index at equal scores
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, kWave);
+      const int oi = __shfl_xor(bi, o, kWave);
+      if (ov > bv || (ov == bv && oi < bi)) bv = ov, bi = oi;
+    }
+    if (bi < E) {
+      chosen_sum += bv;
+      if (lane == 0) open[bi] = -2.f;            // taken
+    }
+    __syncthreads();
+  }
+  const float norm = 1.0f / (chosen_sum + 1e-20f);
+  if (live)
+    for (int e = lane; e < E; e += kWave) w[e] = open[e] == -2.f ? score[e] * norm : 0.f;
+}
+
+extern "C" int ts_route_experts(const float* logits, float* weights, int rows, int experts,
+                                int top, int group_count, int group_keep, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (experts <= 0 || group_count <= 0 || experts % group_count || group_keep <= 0 ||
+      group_keep > group_count || top <= 0 || top > group_keep * (experts / group_count))
+    TS_FAIL("route_experts: %d experts in %d groups, %d kept, cannot give %d", experts,
+            group_count, group_keep, top);
+  const size_t lds = (size_t)4 * (2 * experts + group_count) * sizeof(float);
+  if (lds > 64 * 1024) TS_FAIL("route_experts: %d experts are more than the kernel holds", experts);
+  hipLaunchKernelGGL(route_experts_kernel, dim3((rows + 3) / 4), dim3(256), lds, stream, logits,
+                     weights, rows, experts, top, group_count, group_keep);
+  TS_CHECK_LAUNCH("route_experts");
+  return 0;
+}
+
+// ---------------------------------------------------------------- activation
+// gate_up [rows, E, gate | up] (inner columns each) -> out [rows, E, inner]:
+// g = min(gate, limit), u = clamp(up, -limit, limit), out = g sigmoid(1.702 g) (u + 1) times
+// the token's weight for the expert; zeros (and no reads) where the weight is zero.
+template <typename T>
+__global__ __launch_bounds__(256) void expert_activation_kernel(
+    const T* __restrict__ gate_up, const float* __restrict__ weights, T* __restrict__ out,
+    int64_t total, int E, int inner, float limit) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int64_t te = idx / inner;                 // token * E + expert
+  const int i = (int)(idx % inner);
+  const float w = weights[te];
+  float y = 0.f;
+  if (w != 0.f) {
+    const T* src = gate_up + te * 2 * inner;
+    const float g = fminf(to_f32(src[i]), limit);
+    const float u = fminf(fmaxf(to_f32(src[inner + i]), -limit), limit);
+    y = g / (1.0f + expf(-1.702f * g)) * (u + 1.0f) * w;
+  }
+  out[idx] = from_f32<T>(y);
+}
+
+extern "C" int ts_expert_activation(const void* gate_up, const float* weights, void* out, int type,
+                                    int rows, int experts, int inner, float limit,
+                                    hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (experts <= 0 || inner <= 0) TS_FAIL("expert_activation: bad sizes");
+  const int64_t total = (int64_t)rows * experts * inner;
+  TS_DISPATCH_TYPE(type, T,
+                   hipLaunchKernelGGL(expert_activation_kernel<T>,
+                                      dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                                      (const T*)gate_up, weights, (T*)out, total, experts, inner,
+                                      limit));
+  TS_CHECK_LAUNCH("expert_activation");
+  return 0;
+}

@@ -19,6 +19,7 @@ __device__ __forceinline__ float softplus_f(float v) { return v > 20.f ? v : log
 
 // ---------------------------------------------------------------- convolution
 // u = rows of `proj` (leading dimension ld) from column `col`, `channels` wide.
+// (bias may be null: none.)
 // out_t[c] = silu(bias[c] + sum_k w[c][k] * u_(t - (taps-1) + k)[c]); inputs in front of
 // the sequence are zero, inputs in front of the portion come from state[slot][taps-1][C],
 // whose row j holds the input at position start - (taps-1) + j.
@@ -34,7 +35,7 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(
   const int e = b.entry_of_token[t];
   const int first = b.q_start[e], pos = b.positions[t];
   const float* st = state + (int64_t)b.slot_ids[e] * (taps - 1) * channels;
-  float acc = bias[c];
+  float acc = bias ? bias[c] : 0.f;
   for (int k = 0; k < taps; ++k) {
     const int back = taps - 1 - k;
     if (pos - back < 0) continue;
@@ -88,7 +89,7 @@ __global__ __launch_bounds__(256) void conv_silu_walk_kernel(
     // hist[j], j < taps-1: the input at position start - (taps-1) + j
     if (j < taps - 1 && start - (taps - 1) + j >= 0) hist[j] = st[(int64_t)j * channels + c];
   }
-  const float bc = bias[c];
+  const float bc = bias ? bias[c] : 0.f;
   for (int t = first; t < end; ++t) {
     const float v = proj[(int64_t)t * ld + col + c];
     float acc = bc;

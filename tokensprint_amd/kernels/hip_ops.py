@@ -1029,7 +1029,8 @@ class HipOps:
         if weight.shape[0] != channels or col < 0 or col + channels > ld:
             raise ValueError(f"conv_silu: {channels} channels from column {col} of {ld}, "
                              f"weight {tuple(weight.shape)}")
-        self._check("conv bias", bias, torch.float32, shape=(channels,))
+        if bias is not None:
+            self._check("conv bias", bias, torch.float32, shape=(channels,))
         self._check_state("conv state", state, (taps - 1, channels))
         pos, eot, qs, slots = self._batch_ptrs(batch, T)
         out = torch.empty(T, channels, dtype=torch.float32, device=self.device)
@@ -1094,6 +1095,145 @@ class HipOps:
         self._call(self.lib.ts_gated_group_norm, _ptr(y), _ptr(proj), proj.shape[1], _ptr(norm_w),
                    _ptr(out), _TYPE_CODE[out_dtype], T, inner, groups, c_float(eps),
                    self._stream())
+        return out
+
+    # ------------------------------------------------------------ matrix-state mixers
+    def delta_gates(self, qkv, proj, beta_col, z, z_col, a_log, dt_bias, *, heads, kv_heads, dim,
+                    per_channel):
+        """The gated delta rule's operands.  In place on `qkv` (float32 [T, q | k | v]): every
+        q and k head of `dim` columns becomes a unit vector (eps 1e-6 inside the root), q also
+        times dim^-1/2.  Returns float32 [T, heads + n]: beta = sigmoid(proj[:, beta_col + h]),
+        then g = exp(-exp(a_log[h]) softplus(z[:, z_col + j] + dt_bias[j])) for j over the
+        heads (n = heads) or, `per_channel`, over heads x dim."""
+        self._check("qkv", qkv, torch.float32, ndim=2)
+        T = qkv.shape[0]
+        self._check("proj", proj, torch.float32, ndim=2)
+        self._check("z", z, torch.float32, ndim=2)
+        n = heads * dim if per_channel else heads
+        self._check("A_log", a_log, torch.float32, shape=(heads,))
+        self._check("dt_bias", dt_bias, torch.float32, shape=(n,))
+        if proj.shape[0] != T or z.shape[0] != T:
+            raise ValueError("delta_gates: row counts differ")
+        gates = torch.empty(T, heads + n, dtype=torch.float32, device=self.device)
+        self._call(self.lib.ts_delta_gates, _ptr(qkv), qkv.shape[1], _ptr(proj), proj.shape[1],
+                   int(beta_col), _ptr(z), z.shape[1], int(z_col), _ptr(a_log), _ptr(dt_bias),
+                   _ptr(gates), heads + n, T, heads, kv_heads, dim, int(bool(per_channel)),
+                   self._stream())
+        return gates
+
+    def linear_recurrence(self, x, q_col, k_col, v_col, batch, state, *, heads, kv_heads, dim,
+                          vdim, silu_inputs, decay=None, gates=None, per_channel=False,
+                          delta=False):
+        """Per head and entry, a token at a time: S <- g S; u = v, or (`delta`)
+        u = beta (v - S^T k); S <- S + k u^T; o = S^T q -> float32 [T, heads * vdim].
+        `x` (float32 [T, ld]) holds q and k (kv_heads x dim; head h reads q/k head
+        h // (heads / kv_heads)) and v (heads x vdim) from the given columns, their SiLU taken
+        on the way if `silu_inputs`.  g is `decay` [heads] (fixed), or comes with beta from
+        `gates` ([T, heads + n] as `delta_gates` lays it out, `per_channel`: one g per row of
+        S).  `state` [slots, heads, dim, vdim] float32 carries S from step to step."""
+        self._check("x", x, torch.float32, ndim=2)
+        T, ld = x.shape
+        self._check_state("recurrent state", state, (heads, dim, vdim))
+        if decay is not None:
+            self._check("decay", decay, torch.float32, shape=(heads,))
+        ldg = 0
+        if gates is not None:
+            ldg = heads + (heads * dim if per_channel else heads)
+            self._check("gates", gates, torch.float32, shape=(T, ldg))
+        pos, eot, qs, slots = self._batch_ptrs(batch, T)
+        out = torch.empty(T, heads * vdim, dtype=torch.float32, device=self.device)
+        self._call(self.lib.ts_linear_recurrence, _ptr(x), ld, int(q_col), int(k_col), int(v_col),
+                   _ptr(decay), _ptr(gates), ldg, _ptr(state), _ptr(out), pos, eot, qs, slots, T,
+                   batch.num_entries, heads, kv_heads, dim, vdim, int(bool(silu_inputs)),
+                   int(bool(delta)), int(bool(per_channel)), self._stream())
+        return out
+
+    def norm_gate(self, y, gate_rows, gate_col, norm_w, *, groups, gate, eps, out_dtype):
+        """Each of `groups` equal parts of a row of y (float32) over its root mean square,
+        times norm_w (one value per column of a part, shared by the parts, or one per column
+        of the row), times sigmoid or SiLU (`gate`) of columns [gate_col, gate_col + width) of
+        `gate_rows` (float32)."""
+        self._check("y", y, torch.float32, ndim=2)
+        T, inner = y.shape
+        self._check("gate rows", gate_rows, torch.float32, ndim=2)
+        self._check("norm weight", norm_w, torch.float32, ndim=1)
+        if gate not in ("sigmoid", "silu"):
+            raise ValueError(f"norm_gate: gate {gate!r}; built are sigmoid and silu")
+        if gate_rows.shape[0] != T:
+            raise ValueError("norm_gate: row counts differ")
+        out = torch.empty(T, inner, dtype=out_dtype, device=self.device)
+        self._call(self.lib.ts_norm_gate, _ptr(y), _ptr(gate_rows), gate_rows.shape[1],
+                   int(gate_col), _ptr(norm_w), norm_w.shape[0], _ptr(out), _TYPE_CODE[out_dtype],
+                   T, inner, int(groups), 0 if gate == "sigmoid" else 1, c_float(eps),
+                   self._stream())
+        return out
+
+    # ------------------------------------------------------------ routed experts
+    def route_experts(self, logits, *, top, group_count, group_keep):
+        """Router logits (float32 [T, experts]) -> float32 [T, experts]: a token's weight for
+        each of its `top` experts (softmax score over the chosen scores' sum), zero elsewhere.
+        Only experts of the `group_keep` best of `group_count` groups of neighbours can be
+        chosen (a group's score: its best expert's)."""
+        self._check("router logits", logits, torch.float32, ndim=2)
+        T, E = logits.shape
+        weights = torch.empty(T, E, dtype=torch.float32, device=self.device)
+        self._call(self.lib.ts_route_experts, _ptr(logits), _ptr(weights), T, E, int(top),
+                   int(group_count), int(group_keep), self._stream())
+        return weights
+
+    def expert_activation(self, gate_up, weights, inner, limit, out_dtype):
+        """gate_up [T, experts x (gate | up)] -> [T, experts x inner]: with g = min(gate,
+        limit), u = clamp(up, -limit, limit): g sigmoid(1.702 g) (u + 1) times the token's
+        weight for the expert (zeros where it is zero)."""
+        gate_up = self._rows(gate_up)
+        self._check("gate_up", gate_up, self._FLOATS, ndim=2)
+        T = gate_up.shape[0]
+        self._check("expert weights", weights, torch.float32, ndim=2)
+        E = weights.shape[1]
+        if weights.shape[0] != T or gate_up.shape[1] != E * 2 * inner or out_dtype != gate_up.dtype:
+            raise ValueError(f"expert_activation: gate_up {tuple(gate_up.shape)} for {E} experts "
+                             f"of {inner} columns, out {out_dtype}")
+        out = torch.empty(T, E * inner, dtype=out_dtype, device=self.device)
+        self._call(self.lib.ts_expert_activation, _ptr(gate_up), _ptr(weights), _ptr(out),
+                   _TYPE_CODE[out_dtype], T, E, int(inner), c_float(limit), self._stream())
+        return out
+
+    # ------------------------------------------------------------ sums around the stream
+    def stream_add(self, resid, a, b, row):
+        """In place on the float32 stream: resid += (a + b), then resid += row (float32
+        [width]); each may be None (b only with a)."""
+        self._check("resid", resid, torch.float32, ndim=2)
+        codes = []
+        for name, t in (("a", a), ("b", b)):
+            if t is not None:
+                t = self._rows(t)
+                self._check(name, t, self._FLOATS, shape=resid.shape)
+            codes.append(t)
+        a, b = codes
+        if row is not None:
+            self._check("row", row, torch.float32, shape=(resid.shape[1],))
+        self._call(self.lib.ts_stream_add, _ptr(resid), _ptr(a),
+                   _TYPE_CODE[a.dtype] if a is not None else 0, _ptr(b),
+                   _TYPE_CODE[b.dtype] if b is not None else 0, _ptr(row), resid.shape[0],
+                   resid.shape[1], self._stream())
+
+    def scaled_sum(self, a, scale_a, b, scale_b):
+        """scale_a * a + scale_b * b -> float32."""
+        a, b = self._rows(a), self._rows(b)
+        self._check("a", a, self._FLOATS, ndim=2)
+        self._check("b", b, self._FLOATS, shape=a.shape)
+        out = torch.empty(a.shape, dtype=torch.float32, device=self.device)
+        self._call(self.lib.ts_scaled_sum, _ptr(a), _TYPE_CODE[a.dtype], c_float(scale_a), _ptr(b),
+                   _TYPE_CODE[b.dtype], c_float(scale_b), _ptr(out), a.shape[0], a.shape[1],
+                   self._stream())
+        return out
+
+    def take_columns(self, x, col, count, out_dtype):
+        """Columns [col, col + count) of float32 rows as rows of their own in `out_dtype`."""
+        self._check("x", x, torch.float32, ndim=2)
+        out = torch.empty(x.shape[0], count, dtype=out_dtype, device=self.device)
+        self._call(self.lib.ts_take_columns, _ptr(x), x.shape[1], int(col), int(count), _ptr(out),
+                   _TYPE_CODE[out_dtype], x.shape[0], self._stream())
         return out
 
     # ------------------------------------------------------------ latent attention
