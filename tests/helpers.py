@@ -165,3 +165,106 @@ ZONO_C = zonopel_config(
                        ff=24),
     ])
 ZONO = {"A": (ZONO_A, 11, 4), "B": (ZONO_B, 12, 16), "C": (ZONO_C, 13, 8)}   # cfg, seed, page
+
+
+# ------------------------------------------------------------------ Palelix
+
+
+def palelix_dense(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def palelix_moe(*, ff, limit, experts, top, count, keep):
+    return {"kind": "moe", "expert": {"ff": ff, "limit": limit},
+            "router": {"experts": experts, "top": top, "groups": {"count": count, "keep": keep}}}
+
+
+def palelix_lightning(*, heads, dim, vdim, decay, mlp=None):
+    return {"type": "lightning", "mlp": mlp,
+            "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "decay": list(decay)}}
+
+
+def palelix_delta_sizes(*, heads, kv_heads, dim, vdim, conv, ranks=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv}
+    if ranks is not None:           # of the two-step projections (random weights need them)
+        m.update(decay_rank=ranks[0], gate_rank=ranks[1])
+    return m
+
+
+def palelix_delta(*, mlp=None, **sizes):
+    return {"type": "delta", "mlp": mlp, "mixer": palelix_delta_sizes(**sizes)}
+
+
+def palelix_parallel(*, heads, kv_heads, dim, vdim, rot_dims, base, scale, right, left_scale,
+                     right_scale, mlp=None):
+    return {"type": "parallel", "mlp": mlp,
+            "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+                               "scale": scale, "rot": {"base": base, "dims": rot_dims}},
+                      "right": right, "left_scale": left_scale, "right_scale": right_scale}}
+
+
+def palelix_config(*, width, vocab, eps, layers, loop=None):
+    cfg = {"architecture": "Palelix", "width": width, "vocab": vocab, "norm": {"eps": eps},
+           "layers": layers}
+    if loop is not None:
+        cfg["loop"] = dict(zip(("start", "stop", "times"), loop))
+    return cfg
+
+
+# Three small models that differ in every size and option: loops over the first layers, the
+# last ones, three times, and none; attention whose value size is above, below and equal to
+# its key size, rotated in part and whole, one and several key/value heads; delta rules with
+# shared and own key heads, convolutions of 1 to 4 taps, key sizes that are no multiple of
+# the kernel's eight slices, value sizes above a workgroup's 64 columns; decays that forget
+# at once and almost never; experts in one group, in groups all kept, one expert a token;
+# layers without a feed-forward.
+PALE_A = palelix_config(
+    width=40, vocab=97, eps=1e-5, loop=(0, 2, 3), layers=[
+        palelix_parallel(heads=4, kv_heads=2, dim=12, vdim=20, rot_dims=8, base=10000.0,
+                         scale=0.35, left_scale=0.7, right_scale=1.3,
+                         right=palelix_delta_sizes(heads=3, kv_heads=1, dim=10, vdim=6, conv=2,
+                                                   ranks=(5, 7)),
+                         mlp=palelix_moe(ff=12, limit=0.8, experts=6, top=2, count=3, keep=2)),
+        palelix_lightning(heads=3, dim=6, vdim=9, decay=(0.4, 0.93, 0.999),
+                          mlp=palelix_dense(48)),
+        palelix_delta(heads=2, kv_heads=2, dim=5, vdim=70, conv=4, mlp=None),
+    ])
+PALE_B = palelix_config(
+    width=72, vocab=131, eps=3e-6, loop=(1, 3, 2), layers=[
+        palelix_delta(heads=6, kv_heads=2, dim=20, vdim=12, conv=3,
+                      mlp=palelix_moe(ff=20, limit=2.5, experts=8, top=3, count=1, keep=1)),
+        palelix_lightning(heads=2, dim=24, vdim=16, decay=(0.999, 0.7), mlp=None),
+        palelix_parallel(heads=3, kv_heads=3, dim=16, vdim=8, rot_dims=16, base=300.0,
+                         scale=0.25, left_scale=1.0, right_scale=1.0,
+                         right=palelix_delta_sizes(heads=2, kv_heads=2, dim=9, vdim=24, conv=1,
+                                                   ranks=(8, 4)),
+                         mlp=palelix_dense(100)),
+    ])
+PALE_C = palelix_config(
+    width=32, vocab=64, eps=1e-4, layers=[
+        palelix_lightning(heads=1, dim=16, vdim=8, decay=(0.97,),
+                          mlp=palelix_moe(ff=16, limit=1.2, experts=4, top=1, count=4, keep=4)),
+        palelix_parallel(heads=1, kv_heads=1, dim=8, vdim=8, rot_dims=2, base=50.0, scale=0.5,
+                         left_scale=2.0, right_scale=0.25,
+                         right=palelix_delta_sizes(heads=1, kv_heads=1, dim=8, vdim=8, conv=3,
+                                                   ranks=(3, 3)),
+                         mlp=palelix_moe(ff=8, limit=5.0, experts=5, top=5, count=1, keep=1)),
+        palelix_delta(heads=1, kv_heads=1, dim=32, vdim=4, conv=2, mlp=palelix_dense(24)),
+    ])
+PALE = {"A": (PALE_A, 31, 4), "B": (PALE_B, 32, 16), "C": (PALE_C, 33, 8)}   # cfg, seed, page
+
+
+def write_palelix_model(folder, cfg, seed, dtype, std=0.2, sharpen=4.0):
+    """Random weights, then the softmax attention's query and key weights scaled up, so that
+    its softmax weighs few keys heavily and a key that is lost or seen too early shows."""
+    import json as _json
+    from safetensors.torch import load_file, save_file
+    from tokensprint_amd.weights import write_random_model
+    d = write_random_model(folder, cfg, seed, dtype, std=std)
+    file = next(d.glob("*.safetensors"))
+    tensors = load_file(str(file))
+    for name in tensors:
+        if name.endswith(".left.q") or name.endswith(".left.k"):
+            tensors[name] = (tensors[name].float() * sharpen).to(tensors[name].dtype)
+    save_file(tensors, str(file))
+    return d
