@@ -143,3 +143,22 @@ def test_run_py_serves_a_zonopel_model(gpu_device, tmp_path):
     for _ in range(9):
         tokens.append(int(zonopel_plain.forward(pcfg, w, tokens)[-1].argmax()))
     assert got == tokens[len(prompt):]
+
+
+def test_run_py_serves_a_palelix_model(gpu_device, tmp_path):
+    """The same for Palelix: looped layers, matrix states, routed experts."""
+    from helpers import PALE_B
+    from plain import palelix_plain
+    prompt = random_prompt(21, PALE_B["vocab"], 9)
+    model_dir = tmp_path / "pale-b"
+    proc = run_program(["run.py", "--config-json", config_json(tmp_path, PALE_B),
+                        "--random-weights", "2", "--model-dir", model_dir, "--dtype", "float32",
+                        "--temperature", "0", "--max-tokens", "9", "--ignore-eos", "True",
+                        "--max-num-seqs", "8", "--max-model-len", "256",
+                        "--prompt-ids", ",".join(map(str, prompt))])
+    got = json.loads(proc.stdout.strip().splitlines()[-1])
+    pcfg, w = palelix_plain.read_model_dir(model_dir)
+    tokens = list(prompt)
+    for _ in range(9):
+        tokens.append(int(palelix_plain.forward(pcfg, w, tokens)[-1].argmax()))
+    assert got == tokens[len(prompt):]
