@@ -323,6 +323,49 @@ def compare_configs(s):
     return zono, qwen
 
 
+def palelix_configs(s):
+    """(Palelix, Zonopel) at the width, depth, vocabulary and number of matrix parameters of
+    the size `s`.  Palelix: gated delta rule, lightning attention, gated delta rule, softmax
+    attention beside a delta rule with decays per key channel, twice; routed experts (8, of
+    which a token uses 2, in 4 groups of which 2 are kept) in every second layer and a dense
+    feed-forward in the others; the experts' inner size takes up what is left."""
+    import math
+    from tokensprint_amd.weights.random_init import declared_tensors
+    hd, heads, kv = s["head_dim"], s["heads"], s["kv_heads"]
+
+    def moe(ff):
+        return {"kind": "moe", "expert": {"ff": ff, "limit": 7.0},
+                "router": {"experts": 8, "top": 2, "groups": {"count": 4, "keep": 2}}}
+
+    def layers(expert_ff):
+        delta = {"type": "delta", "mixer": {"heads": heads, "kv_heads": kv, "dim": hd,
+                                            "vdim": hd, "conv": 4}}
+        lightning = {"type": "lightning", "mixer": {
+            "heads": heads, "dim": hd, "vdim": hd,
+            "decay": [1.0 - 2.0 ** (-(2 + 6 * i / max(heads - 1, 1))) for i in range(heads)]}}
+        parallel = {"type": "parallel", "mixer": {
+            "left": {"heads": heads, "kv_heads": kv, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+                     "rot": {"base": 1e6, "dims": hd // 2}},
+            "right": {"heads": kv, "kv_heads": kv, "dim": hd // 2, "vdim": hd, "conv": 4,
+                      "decay_rank": 64, "gate_rank": 64},
+            "left_scale": 1.0, "right_scale": 1.0}}
+        kinds = [delta, lightning, delta, parallel]
+        return [dict(kinds[i % 4], mlp=moe(expert_ff) if i % 2 else
+                     {"kind": "dense", "ff": s["ff"]}) for i in range(s["layers"])]
+
+    def config(expert_ff):
+        return {"architecture": "Palelix", "width": s["width"], "vocab": s["vocab"],
+                "norm": {"eps": 1e-6}, "layers": layers(expert_ff)}
+
+    def count(raw):
+        return sum(math.prod(d.shape) for d in declared_tensors(raw).values())
+    zono = compare_configs(s)[0]
+    spare = count(zono) - count(config(64))
+    moe_layers = s["layers"] // 2
+    ff = 64 + max(0, round(spare / (3 * s["width"] * 8 * moe_layers) / 64)) * 64
+    return config(ff), zono
+
+
 class TimedOps:
     """Wraps a kernel provider: every call of one of its operations is bracketed by events,
     and `seconds` sums them per operation name (an eager step's kernels, one by one)."""
@@ -383,12 +426,15 @@ def op_times(model, page, entries_of, reps=3):
 
 
 def zonopel_profile_step(args) -> int:
-    """Four eager steps of the Zonopel model of `--compare-size` (default 1b-layers): a
-    2,048-token prompt, or a decode step of eight requests at 2,048 tokens; for a profiler."""
+    """Four eager steps of the Zonopel (or, `--profile-palelix`, the Palelix) model of
+    `--compare-size` (default 1b-layers): a 2,048-token prompt, or a decode step of eight
+    requests at 2,048 tokens; for a profiler."""
     import torch
     from tokensprint_amd.engine.assemble import random_model
     from tokensprint_amd.engine.runner import ModelRunner
-    zono, _ = compare_configs(COMPARE_SIZES[args.compare_size or "1b-layers"])
+    size = COMPARE_SIZES[args.compare_size or "1b-layers"]
+    zono = palelix_configs(size)[0] if args.profile_palelix else compare_configs(size)[0]
+    args.profile_zonopel = args.profile_zonopel or args.profile_palelix
     _, model = random_model(zono, 0, args.dtype, "cuda:0")
     make = prefill_entries(2048) if args.profile_zonopel == "prefill" else decode_entries(8, 2048)
     lengths = make(None)
@@ -410,12 +456,15 @@ def zonopel_compare(args) -> int:
     import torch
     from tokensprint_amd.engine.assemble import random_model
     page, T, b, ctx = 16, 2048, 8, 2048
-    out = {"metric": "zonopel beside qwen3 at equal sizes (random weights, bf16)", "sizes": {}}
+    pair = ("palelix", "zonopel") if args.compare_palelix else ("zonopel", "qwen3")
+    out = {"metric": f"{pair[0]} beside {pair[1]} at equal sizes (random weights, bf16)",
+           "sizes": {}}
     for name, size in COMPARE_SIZES.items():
         if args.compare_size and name != args.compare_size:
             continue
         row = {}
-        for design, raw in zip(("zonopel", "qwen3"), compare_configs(size)):
+        configs = palelix_configs(size) if args.compare_palelix else compare_configs(size)
+        for design, raw in zip(pair, configs):
             _, model = random_model(raw, 0, args.dtype, "cuda:0")
             vocab = size["vocab"]
             _, engine = make_engine(raw, args.dtype, None, 1, 4096, T, page, model=model)
@@ -467,7 +516,12 @@ def main() -> int:
     ap.add_argument("--compare-zonopel", action="store_true",
                     help="instead of the benchmark: Zonopel beside Qwen3 at equal sizes "
                          "(prefill, decode, time per kind of kernel); prints its own line")
-    ap.add_argument("--compare-size", default=None, help="with --compare-zonopel: one size only")
+    ap.add_argument("--compare-palelix", action="store_true",
+                    help="instead of the benchmark: Palelix beside Zonopel at equal sizes "
+                         "(prefill and decode throughput, time per kind of kernel)")
+    ap.add_argument("--profile-palelix", default=None, choices=["prefill", "decode"],
+                    help="as --profile-zonopel, for the Palelix model of --compare-size")
+    ap.add_argument("--compare-size", default=None, help="with --compare-...: one size only")
     ap.add_argument("--profile-zonopel", default=None, choices=["prefill", "decode"],
                     help="instead of the benchmark: four eager steps of the Zonopel model of "
                          "--compare-size, for a profiler")
@@ -479,9 +533,9 @@ def main() -> int:
     import torch
     from tokensprint_amd.config import load_named_config
 
-    if args.profile_zonopel:
+    if args.profile_zonopel or args.profile_palelix:
         return zonopel_profile_step(args)
-    if args.compare_zonopel:
+    if args.compare_zonopel or args.compare_palelix:
         return zonopel_compare(args)
     raw = load_named_config(args.model)
     full_layers = raw["num_hidden_layers"]

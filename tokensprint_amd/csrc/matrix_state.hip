@@ -40,156 +40,237 @@ struct RecurrenceArgs {
 
 constexpr int kRecSlices = 8;              // lanes that share a column's dot products
 constexpr int kRecThreads = 128;
-constexpr int kRecPerThread = 4;           // columns a thread owns
-constexpr int kRecBlockCols = kRecThreads / kRecSlices * kRecPerThread;   // 64
+constexpr int kRecGroups = kRecThreads / kRecSlices;   // 16 groups of columns a workgroup
 constexpr int kRecStage = 16;              // tokens staged in LDS at a time
 
-// A workgroup serves one (entry, head, 64 columns of P) and walks the entry's tokens in
-// order.  Thread (cg, s) = (tid / 8, tid % 8) keeps rows s, s + 8, ... of four columns in
-// registers; sixteen tokens' q, k, the workgroup's columns of v, and the gates are staged in
-// LDS by all threads together; a column's dot products over the rows are added over the
-// eight lanes that share it, in one fixed butterfly.
-template <int NI, bool DELTA, bool PER_ROW>
+// Sum over the eight neighbouring lanes that share a column; every one of them gets it.  Two
+// exchanges inside a quad and one with the mirrored lane of the eight, all three in the
+// vector pipeline (a shuffle through LDS costs a round trip each, on the recurrence's chain).
+__device__ __forceinline__ float sum8(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true));
+  return v;
+}
+
+template <int NI>
+__device__ __forceinline__ void read_rows(const float* p, float (&r)[NI]) {
+  if constexpr (NI % 4 == 0) {
+#pragma unroll
+    for (int j = 0; j < NI / 4; ++j) {
+      const float4 v = reinterpret_cast<const float4*>(p)[j];
+      r[4 * j] = v.x, r[4 * j + 1] = v.y, r[4 * j + 2] = v.z, r[4 * j + 3] = v.w;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < NI; ++j) r[j] = p[j];
+  }
+}
+
+// A workgroup serves one (entry, head, 16 CPT columns of P) and walks the entry's tokens in
+// order.  Thread (cg, s) = (tid / 8, tid % 8) keeps rows [s NI, (s + 1) NI) of CPT columns in
+// registers; a column's dot products over the rows are added over the eight lanes that share
+// it, in one fixed order whatever CPT is, so the result does not depend on how a launch is
+// shaped.  Sixteen tokens' q, k, the workgroup's columns of v, and the gates are staged in
+// one of two LDS buffers (rows padded to 8 NI, so a thread's rows come in 16-byte reads)
+// while the sixteen before them are walked.
+template <int NI, int CPT, bool DELTA, bool PER_ROW>
 __global__ __launch_bounds__(kRecThreads) void recurrence_kernel(RecurrenceArgs a) {
-  extern __shared__ float lds[];
+  extern __shared__ __align__(16) float lds[];
+  constexpr int NP = kRecSlices * NI;                // padded rows
+  constexpr int BC = kRecGroups * CPT;               // columns of the workgroup
+  constexpr int kQ = 0, kK = kRecStage * NP, kG = 2 * kRecStage * NP;
+  constexpr int kV = kG + kRecStage * (PER_ROW ? NP : 1);
+  constexpr int kB = kV + kRecStage * BC;
+  constexpr int kBuf = (kB + kRecStage + 3) / 4 * 4;
+  constexpr int VPT = kRecStage * BC / kRecThreads;  // values of v a thread stages: 2 CPT
   const int N = a.N;
-  float* q_s = lds;                                  // [stage][N]
-  float* k_s = q_s + kRecStage * N;                  // [stage][N]
-  float* g_s = k_s + kRecStage * N;                  // [stage][N] (PER_ROW) or [stage]
-  float* v_s = g_s + kRecStage * (PER_ROW ? N : 1);  // [stage][64]
-  float* b_s = v_s + kRecStage * kRecBlockCols;      // [stage]: beta
   const int h = blockIdx.x, e = blockIdx.y;
   const int s = threadIdx.x % kRecSlices, cg = threadIdx.x / kRecSlices;
-  const int col0 = blockIdx.z * kRecBlockCols;
-  const int p0 = col0 + cg * kRecPerThread;
+  const int col0 = blockIdx.z * BC;
+  const int p0 = col0 + cg * CPT;
   const int hk = h / (a.heads / a.kv_heads);
   const int first = a.b.q_start[e], end = a.b.q_start[e + 1];
   float* st = a.state + ((int64_t)a.b.slot_ids[e] * a.heads + h) * N * a.P;
   const bool fresh = a.b.positions[first] == 0;
-  float S[NI][kRecPerThread];
+  float S[NI][CPT];
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
-    const int n = s + kRecSlices * i;
+    const int n = s * NI + i;
 #pragma unroll
-    for (int c = 0; c < kRecPerThread; ++c)
+    for (int c = 0; c < CPT; ++c)
       S[i][c] = (!fresh && n < N && p0 + c < a.P) ? st[(int64_t)n * a.P + p0 + c] : 0.f;
   }
   const float fixed_decay = a.decay ? a.decay[h] : 1.f;
   const int inner = a.heads * a.P;
+  for (int i = threadIdx.x; i < 2 * kBuf; i += kRecThreads) lds[i] = 0.f;   // the rows' padding
+  __syncthreads();
 
-  for (int t0 = first; t0 < end; t0 += kRecStage) {
+  // a stage's operands: from memory into registers (fetch), from there into a buffer (commit)
+  float pq[NI], pk[NI], pg[PER_ROW ? NI : 1], pv[VPT], pbeta = 0.f, pgate = 1.f;
+  auto fetch = [&](int t0) {
     const int nt = min(kRecStage, end - t0);
-    __syncthreads();                                  // the stage before has been walked
-    for (int i = threadIdx.x; i < nt * N; i += kRecThreads) {
-      const int tt = i / N, n = i % N;
-      const float* row = a.x + (int64_t)(t0 + tt) * a.ld;
-      float qv = row[a.q_col + hk * N + n], kv = row[a.k_col + hk * N + n];
-      if (a.silu) qv = silu_f(qv), kv = silu_f(kv);
-      q_s[i] = qv;
-      k_s[i] = kv;
-      if (PER_ROW) g_s[i] = a.gates[(int64_t)(t0 + tt) * a.ldg + a.heads + h * N + n];
-    }
-    for (int i = threadIdx.x; i < kRecStage * kRecBlockCols; i += kRecThreads) {
-      const int tt = i / kRecBlockCols, c = i % kRecBlockCols;
-      float v = 0.f;
-      if (tt < nt && col0 + c < a.P) {
-        v = a.x[(int64_t)(t0 + tt) * a.ld + a.v_col + h * a.P + col0 + c];
-        if (a.silu) v = silu_f(v);
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int i = j * kRecThreads + threadIdx.x;
+      const int tt = i / N, n = i - tt * N;
+      pq[j] = pk[j] = 0.f;
+      if (PER_ROW) pg[j] = 0.f;
+      if (tt < nt) {
+        const float* row = a.x + (int64_t)(t0 + tt) * a.ld;
+        pq[j] = row[a.q_col + hk * N + n];
+        pk[j] = row[a.k_col + hk * N + n];
+        if (PER_ROW) pg[j] = a.gates[(int64_t)(t0 + tt) * a.ldg + a.heads + h * N + n];
       }
-      v_s[i] = v;
+    }
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+      const int i = j * kRecThreads + threadIdx.x;
+      const int tt = i / BC, c = i % BC;
+      pv[j] = (tt < nt && col0 + c < a.P)
+          ? a.x[(int64_t)(t0 + tt) * a.ld + a.v_col + h * a.P + col0 + c] : 0.f;
     }
     if (threadIdx.x < nt) {
       const float* gr = a.gates ? a.gates + (int64_t)(t0 + threadIdx.x) * a.ldg : nullptr;
-      if (DELTA) b_s[threadIdx.x] = gr[h];
-      if (!PER_ROW) g_s[threadIdx.x] = gr ? gr[a.heads + h] : fixed_decay;
+      if (DELTA) pbeta = gr[h];
+      if (!PER_ROW) pgate = gr ? gr[a.heads + h] : fixed_decay;
     }
-    __syncthreads();
+  };
+  auto commit = [&](float* buf) {
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int i = j * kRecThreads + threadIdx.x;
+      const int tt = i / N, n = i - tt * N;
+      if (tt < kRecStage) {
+        buf[kQ + tt * NP + n] = a.silu ? silu_f(pq[j]) : pq[j];
+        buf[kK + tt * NP + n] = a.silu ? silu_f(pk[j]) : pk[j];
+        if (PER_ROW) buf[kG + tt * NP + n] = pg[j];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < VPT; ++j)
+      buf[kV + j * kRecThreads + threadIdx.x] = a.silu ? silu_f(pv[j]) : pv[j];
+    if (threadIdx.x < kRecStage) {
+      if (DELTA) buf[kB + threadIdx.x] = pbeta;
+      if (!PER_ROW) buf[kG + threadIdx.x] = pgate;
+    }
+  };
+
+  fetch(first);
+  commit(lds);
+  __syncthreads();
+  int which = 0;
+  for (int t0 = first; t0 < end; t0 += kRecStage, which ^= 1) {
+    const int nt = min(kRecStage, end - t0);
+    const bool more = t0 + kRecStage < end;
+    if (more) fetch(t0 + kRecStage);
+    const float* buf = lds + which * kBuf;
     for (int tt = 0; tt < nt; ++tt) {
-      float u[kRecPerThread], acc[kRecPerThread];
+      float kr[NI], u[CPT], acc[CPT];
+      read_rows<NI>(buf + kK + tt * NP + s * NI, kr);
 #pragma unroll
-      for (int c = 0; c < kRecPerThread; ++c) u[c] = v_s[tt * kRecBlockCols + cg * kRecPerThread + c];
-      const float g_all = PER_ROW ? 1.f : g_s[tt];
+      for (int c = 0; c < CPT; ++c) u[c] = buf[kV + tt * BC + cg * CPT + c];
+      const float g_all = PER_ROW ? 1.f : buf[kG + tt];
       if (DELTA) {
-        float pred[kRecPerThread];
+        float gr[NI];
+        if constexpr (PER_ROW) read_rows<NI>(buf + kG + tt * NP + s * NI, gr);
+        float pred[CPT][2];
 #pragma unroll
-        for (int c = 0; c < kRecPerThread; ++c) pred[c] = 0.f;
+        for (int c = 0; c < CPT; ++c) pred[c][0] = pred[c][1] = 0.f;
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-          const int n = s + kRecSlices * i;
-          const float kv = n < N ? k_s[tt * N + n] : 0.f;
-          const float g = PER_ROW ? (n < N ? g_s[tt * N + n] : 1.f) : g_all;
+          const float g = PER_ROW ? gr[i] : g_all;
 #pragma unroll
-          for (int c = 0; c < kRecPerThread; ++c) {
+          for (int c = 0; c < CPT; ++c) {
             S[i][c] *= g;
-            pred[c] = fmaf(S[i][c], kv, pred[c]);
+            pred[c][i & 1] = fmaf(S[i][c], kr[i], pred[c][i & 1]);
           }
         }
-        const float beta = b_s[tt];
+        const float beta = buf[kB + tt];
 #pragma unroll
-        for (int c = 0; c < kRecPerThread; ++c) {
-          pred[c] += __shfl_xor(pred[c], 1, kWave);
-          pred[c] += __shfl_xor(pred[c], 2, kWave);
-          pred[c] += __shfl_xor(pred[c], 4, kWave);
-          u[c] = beta * (u[c] - pred[c]);
-        }
+        for (int c = 0; c < CPT; ++c) u[c] = beta * (u[c] - sum8(pred[c][0] + pred[c][1]));
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+#pragma unroll
+          for (int c = 0; c < CPT; ++c) S[i][c] = fmaf(kr[i], u[c], S[i][c]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+#pragma unroll
+          for (int c = 0; c < CPT; ++c) S[i][c] = fmaf(g_all, S[i][c], kr[i] * u[c]);
       }
+      float qr[NI];
+      read_rows<NI>(buf + kQ + tt * NP + s * NI, qr);
 #pragma unroll
-      for (int c = 0; c < kRecPerThread; ++c) acc[c] = 0.f;
+      for (int c = 0; c < CPT; ++c) {
+        float a0 = 0.f, a1 = 0.f;
 #pragma unroll
-      for (int i = 0; i < NI; ++i) {
-        const int n = s + kRecSlices * i;
-        const float kv = n < N ? k_s[tt * N + n] : 0.f;
-        const float qv = n < N ? q_s[tt * N + n] : 0.f;
-#pragma unroll
-        for (int c = 0; c < kRecPerThread; ++c) {
-          if (DELTA) S[i][c] = fmaf(kv, u[c], S[i][c]);
-          else S[i][c] = fmaf(g_all, S[i][c], kv * u[c]);
-          acc[c] = fmaf(S[i][c], qv, acc[c]);
+        for (int i = 0; i < NI; i += 2) {
+          a0 = fmaf(S[i][c], qr[i], a0);
+          a1 = fmaf(S[i + 1][c], qr[i + 1], a1);
         }
-      }
-#pragma unroll
-      for (int c = 0; c < kRecPerThread; ++c) {
-        acc[c] += __shfl_xor(acc[c], 1, kWave);
-        acc[c] += __shfl_xor(acc[c], 2, kWave);
-        acc[c] += __shfl_xor(acc[c], 4, kWave);
+        acc[c] = sum8(a0 + a1);
         if (s == 0 && p0 + c < a.P) a.out[(int64_t)(t0 + tt) * inner + h * a.P + p0 + c] = acc[c];
       }
     }
+    if (more) commit(lds + (which ^ 1) * kBuf);
+    __syncthreads();
   }
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
-    const int n = s + kRecSlices * i;
+    const int n = s * NI + i;
 #pragma unroll
-    for (int c = 0; c < kRecPerThread; ++c)
+    for (int c = 0; c < CPT; ++c)
       if (n < N && p0 + c < a.P) st[(int64_t)n * a.P + p0 + c] = S[i][c];
   }
 }
 
-template <int NI>
-static void launch_recurrence(const RecurrenceArgs& a, int num_entries, bool delta, bool per_row,
-                              hipStream_t stream) {
-  const dim3 grid(a.heads, num_entries, (a.P + kRecBlockCols - 1) / kRecBlockCols);
+template <int NI, int CPT>
+static int launch_recurrence_cols(const RecurrenceArgs& a, int num_entries, bool delta, bool per_row,
+                                  hipStream_t stream) {
+  constexpr int NP = kRecSlices * NI, BC = kRecGroups * CPT;
+  const dim3 grid(a.heads, num_entries, (a.P + BC - 1) / BC);
   const dim3 block(kRecThreads);
-  const size_t lds = (size_t)kRecStage * (2 * a.N + (per_row ? a.N : 1) + kRecBlockCols + 1) *
-                     sizeof(float);
+  const int buf = (kRecStage * (2 * NP + (per_row ? NP : 1) + BC + 1) + 3) / 4 * 4;
+  const size_t lds = (size_t)2 * buf * sizeof(float);
+  const void* fn = delta && per_row ? (const void*)recurrence_kernel<NI, CPT, true, true>
+                   : delta          ? (const void*)recurrence_kernel<NI, CPT, true, false>
+                                    : (const void*)recurrence_kernel<NI, CPT, false, false>;
+  if (lds > 64 * 1024 &&
+      hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return -1;
   if (delta && per_row)
-    hipLaunchKernelGGL((recurrence_kernel<NI, true, true>), grid, block, lds, stream, a);
+    hipLaunchKernelGGL((recurrence_kernel<NI, CPT, true, true>), grid, block, lds, stream, a);
   else if (delta)
-    hipLaunchKernelGGL((recurrence_kernel<NI, true, false>), grid, block, lds, stream, a);
+    hipLaunchKernelGGL((recurrence_kernel<NI, CPT, true, false>), grid, block, lds, stream, a);
   else
-    hipLaunchKernelGGL((recurrence_kernel<NI, false, false>), grid, block, lds, stream, a);
+    hipLaunchKernelGGL((recurrence_kernel<NI, CPT, false, false>), grid, block, lds, stream, a);
+  return 0;
+}
+
+// Four columns a thread where the launch has workgroups enough without (a step of many
+// entries streams its states in wider rows); one column a thread where a few entries' long
+// portions are walked, which is then sixteen times the workgroups and a quarter of the
+// chain a token.
+template <int NI>
+static int launch_recurrence(const RecurrenceArgs& a, int num_entries, bool delta, bool per_row,
+                             bool narrow, hipStream_t stream) {
+  return narrow ? launch_recurrence_cols<NI, 1>(a, num_entries, delta, per_row, stream)
+                : launch_recurrence_cols<NI, 4>(a, num_entries, delta, per_row, stream);
 }
 
 // x [T, ld] float32 holds q, k (kv_heads x N each) and v (heads x P) at the given columns
 // (`silu`: their SiLU is taken as they are read).  `decay` [heads]: fixed decays, or null and
 // `gates` [T, ldg] holds beta (heads; read by the delta rule only) and then the decays, one
-// per head or (`per_row`) one per head and row of S.  out [T, heads*P].
+// per head or (`per_row`) one per head and row of S.  out [T, heads*P].  `max_q_len`: the
+// most tokens an entry brings (it chooses the launch's shape, never a result).
 extern "C" int ts_linear_recurrence(const float* x, int ld, int q_col, int k_col, int v_col,
                                     const float* decay, const float* gates, int ldg, float* state,
                                     float* out, const int* positions, const int* entry_of_token,
                                     const int* q_start, const int* slot_ids, int num_tokens,
-                                    int num_entries, int heads, int kv_heads, int N, int P,
-                                    int silu, int delta, int per_row, hipStream_t stream) {
+                                    int num_entries, int max_q_len, int heads, int kv_heads,
+                                    int N, int P, int silu, int delta, int per_row,
+                                    hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || N <= 0 || P <= 0)
     TS_FAIL("linear_recurrence: bad sizes heads=%d kv_heads=%d dim=%d vdim=%d", heads, kv_heads, N, P);
@@ -208,11 +289,15 @@ extern "C" int ts_linear_recurrence(const float* x, int ld, int q_col, int k_col
                    BatchView{positions, entry_of_token, q_start, slot_ids},
                    ld, q_col, k_col, v_col, ldg, heads, kv_heads, N, P, silu};
   const int ni = (N + kRecSlices - 1) / kRecSlices;
-  if (ni <= 2) launch_recurrence<2>(a, num_entries, delta, per_row, stream);
-  else if (ni <= 4) launch_recurrence<4>(a, num_entries, delta, per_row, stream);
-  else if (ni <= 8) launch_recurrence<8>(a, num_entries, delta, per_row, stream);
-  else if (ni <= 16) launch_recurrence<16>(a, num_entries, delta, per_row, stream);
-  else launch_recurrence<32>(a, num_entries, delta, per_row, stream);
+  const int64_t wide_groups = (int64_t)heads * num_entries * ((P + 4 * kRecGroups - 1) / (4 * kRecGroups));
+  const bool narrow = max_q_len >= 8 && wide_groups < 1024;
+  int rc;
+  if (ni <= 2) rc = launch_recurrence<2>(a, num_entries, delta, per_row, narrow, stream);
+  else if (ni <= 4) rc = launch_recurrence<4>(a, num_entries, delta, per_row, narrow, stream);
+  else if (ni <= 8) rc = launch_recurrence<8>(a, num_entries, delta, per_row, narrow, stream);
+  else if (ni <= 16) rc = launch_recurrence<16>(a, num_entries, delta, per_row, narrow, stream);
+  else rc = launch_recurrence<32>(a, num_entries, delta, per_row, true, stream);   // (registers)
+  if (rc != 0) TS_FAIL("linear_recurrence: %d key channels need more LDS than the device gives", N);
   TS_CHECK_LAUNCH("linear_recurrence");
   return 0;
 }

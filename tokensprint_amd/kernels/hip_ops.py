@@ -1144,7 +1144,8 @@ class HipOps:
         out = torch.empty(T, heads * vdim, dtype=torch.float32, device=self.device)
         self._call(self.lib.ts_linear_recurrence, _ptr(x), ld, int(q_col), int(k_col), int(v_col),
                    _ptr(decay), _ptr(gates), ldg, _ptr(state), _ptr(out), pos, eot, qs, slots, T,
-                   batch.num_entries, heads, kv_heads, dim, vdim, int(bool(silu_inputs)),
+                   batch.num_entries, int(batch.max_q_len), heads, kv_heads, dim, vdim,
+                   int(bool(silu_inputs)),
                    int(bool(delta)), int(bool(per_channel)), self._stream())
         return out
 
