@@ -98,6 +98,35 @@ def test_recurrence_over_steps_with_stale_state(gpu_device, mode, heads, kv_head
         close(st, st_ref, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("mode", ["fixed", "per_head_plain"])
+@pytest.mark.parametrize("heads, dim, vdim", [(4, 16, 64), (3, 10, 6), (2, 128, 70)])
+def test_long_portions_run_in_chunks(gpu_device, mode, heads, dim, vdim):
+    """Without the delta rule portions beyond 128 tokens are cut into chunks of 64 that run
+    side by side; beside them short portions and single tokens, states carried on."""
+    ops = load_hip_ops(gpu_device)
+    qk, inner = heads * dim, heads * vdim
+    scene = Scene(gpu_device, SlotStateNeed((heads, dim, vdim), torch.float32, "s"), 8, 4,
+                  num_pages=200)
+    st = scene.view.states["s"]
+    st.fill_(3.0)
+    st_ref = st.clone()
+    decay = (0.9 + 0.1 * torch.rand(heads, generator=torch.Generator().manual_seed(1))).to(gpu_device)
+    for i, spans in enumerate([[300, 1, 131, 5], [1, 1, 1, 1], [200, 3, 0, 129]]):
+        batch = scene.step(spans)
+        T = batch.num_tokens
+        x = rnd((T, 2 * qk + inner), 10 + i, 0.5).to(gpu_device)
+        kw = dict(heads=heads, kv_heads=heads, dim=dim, vdim=vdim)
+        if mode == "fixed":
+            kw.update(silu_inputs=True, decay=decay)
+        else:
+            gates = 0.9 + 0.1 * torch.rand(T, 2 * heads, generator=torch.Generator().manual_seed(i))
+            kw.update(silu_inputs=False, gates=gates.to(gpu_device))
+        got = ops.linear_recurrence(x, 0, qk, 2 * qk, batch, st, **kw)
+        want = REF.linear_recurrence(x, 0, qk, 2 * qk, batch, st_ref, **kw)
+        close(got, want, rtol=2e-4, atol=2e-4)
+        close(st, st_ref, rtol=2e-4, atol=2e-4)
+
+
 @pytest.mark.parametrize("delta", [False, True])
 def test_a_write_is_remembered_over_hundreds_of_steps_and_forgotten(gpu_device, delta):
     """One token writes a value under a key; 300 tokens later, alone in their steps, a query

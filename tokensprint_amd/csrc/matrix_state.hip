@@ -36,7 +36,19 @@ struct RecurrenceArgs {
   float* out;            // [T, heads*P]
   BatchView b;
   int ld, q_col, k_col, v_col, ldg, heads, kv_heads, N, P, silu;
+  const int* chunks;        // [num_chunks, 3]: first token, one past the last, entry
+  const int* entry_chunks;  // [B + 1]: the chunks of entry e are [entry_chunks[e], entry_chunks[e+1])
+  float* chunk_state;       // [num_chunks, heads, N, P]: local contribution, then start state
+  float* chunk_decay;       // [num_chunks, heads]
 };
+
+// Without the delta rule the recurrence is linear in S, and a long portion is cut into
+// chunks of 64 tokens that run side by side, in three launches: every chunk's recurrence
+// from an empty state (its own contribution and the product of its decays, kRecLocal); per
+// entry, the state in front of every chunk, one after the other, and the state the portion
+// leaves (combine); every chunk once more from its true start state, now writing o
+// (kRecOutput).  Twice the arithmetic, a sixty-fourth of the chain.
+constexpr int kRecWhole = 0, kRecLocal = 1, kRecOutput = 2;
 
 constexpr int kRecSlices = 8;              // lanes that share a column's dot products
 constexpr int kRecThreads = 128;
@@ -74,7 +86,7 @@ __device__ __forceinline__ void read_rows(const float* p, float (&r)[NI]) {
 // shaped.  Sixteen tokens' q, k, the workgroup's columns of v, and the gates are staged in
 // one of two LDS buffers (rows padded to 8 NI, so a thread's rows come in 16-byte reads)
 // while the sixteen before them are walked.
-template <int NI, int CPT, bool DELTA, bool PER_ROW>
+template <int NI, int CPT, bool DELTA, bool PER_ROW, int MODE = kRecWhole>
 __global__ __launch_bounds__(kRecThreads) void recurrence_kernel(RecurrenceArgs a) {
   extern __shared__ __align__(16) float lds[];
   constexpr int NP = kRecSlices * NI;                // padded rows
@@ -85,14 +97,26 @@ __global__ __launch_bounds__(kRecThreads) void recurrence_kernel(RecurrenceArgs 
   constexpr int kBuf = (kB + kRecStage + 3) / 4 * 4;
   constexpr int VPT = kRecStage * BC / kRecThreads;  // values of v a thread stages: 2 CPT
   const int N = a.N;
-  const int h = blockIdx.x, e = blockIdx.y;
+  const int h = blockIdx.x;
   const int s = threadIdx.x % kRecSlices, cg = threadIdx.x / kRecSlices;
   const int col0 = blockIdx.z * BC;
   const int p0 = col0 + cg * CPT;
   const int hk = h / (a.heads / a.kv_heads);
-  const int first = a.b.q_start[e], end = a.b.q_start[e + 1];
-  float* st = a.state + ((int64_t)a.b.slot_ids[e] * a.heads + h) * N * a.P;
-  const bool fresh = a.b.positions[first] == 0;
+  int first, end, e;
+  if (MODE == kRecWhole) {
+    e = blockIdx.y;
+    first = a.b.q_start[e];
+    end = a.b.q_start[e + 1];
+  } else {
+    first = a.chunks[3 * blockIdx.y];
+    end = a.chunks[3 * blockIdx.y + 1];
+    e = a.chunks[3 * blockIdx.y + 2];
+  }
+  float* st = MODE == kRecWhole
+      ? a.state + ((int64_t)a.b.slot_ids[e] * a.heads + h) * N * a.P
+      : a.chunk_state + ((int64_t)blockIdx.y * a.heads + h) * N * a.P;
+  const bool fresh = MODE == kRecLocal || (MODE == kRecWhole && a.b.positions[first] == 0);
+  float total_decay = 1.f;
   float S[NI][CPT];
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
@@ -199,6 +223,10 @@ __global__ __launch_bounds__(kRecThreads) void recurrence_kernel(RecurrenceArgs 
 #pragma unroll
           for (int c = 0; c < CPT; ++c) S[i][c] = fmaf(g_all, S[i][c], kr[i] * u[c]);
       }
+      if (MODE == kRecLocal) {
+        total_decay *= g_all;
+        continue;
+      }
       float qr[NI];
       read_rows<NI>(buf + kQ + tt * NP + s * NI, qr);
 #pragma unroll
@@ -216,6 +244,7 @@ __global__ __launch_bounds__(kRecThreads) void recurrence_kernel(RecurrenceArgs 
     if (more) commit(lds + (which ^ 1) * kBuf);
     __syncthreads();
   }
+  if (MODE == kRecOutput) return;
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
     const int n = s * NI + i;
@@ -223,6 +252,42 @@ __global__ __launch_bounds__(kRecThreads) void recurrence_kernel(RecurrenceArgs 
     for (int c = 0; c < CPT; ++c)
       if (n < N && p0 + c < a.P) st[(int64_t)n * a.P + p0 + c] = S[i][c];
   }
+  if (MODE == kRecLocal && blockIdx.z == 0 && threadIdx.x == 0)
+    a.chunk_decay[(int64_t)blockIdx.y * a.heads + h] = total_decay;
+}
+
+// A thread per element of S and (head, entry): walks the entry's chunks in order.
+// chunk_state[c] holds the chunk's own contribution and receives the state in front of the
+// chunk; the state behind the last chunk goes to the request's slot.
+__global__ __launch_bounds__(256) void recurrence_combine_kernel(RecurrenceArgs a) {
+  const int h = blockIdx.x, e = blockIdx.y;
+  const int idx = blockIdx.z * blockDim.x + threadIdx.x;
+  const int size = a.N * a.P;
+  if (idx >= size) return;
+  float* st = a.state + ((int64_t)a.b.slot_ids[e] * a.heads + h) * size;
+  float S = a.b.positions[a.b.q_start[e]] == 0 ? 0.f : st[idx];
+  for (int c = a.entry_chunks[e]; c < a.entry_chunks[e + 1]; ++c) {
+    float* cs = a.chunk_state + ((int64_t)c * a.heads + h) * size;
+    const float local = cs[idx];
+    cs[idx] = S;
+    S = fmaf(a.chunk_decay[(int64_t)c * a.heads + h], S, local);
+  }
+  st[idx] = S;
+}
+
+template <int NI, int CPT>
+static void launch_recurrence_chunked(const RecurrenceArgs& a, int num_entries, int num_chunks,
+                                      hipStream_t stream) {
+  constexpr int NP = kRecSlices * NI, BC = kRecGroups * CPT;
+  const dim3 grid(a.heads, num_chunks, (a.P + BC - 1) / BC);
+  const int buf = (kRecStage * (2 * NP + 1 + BC + 1) + 3) / 4 * 4;
+  const size_t lds = (size_t)2 * buf * sizeof(float);
+  hipLaunchKernelGGL((recurrence_kernel<NI, CPT, false, false, kRecLocal>), grid,
+                     dim3(kRecThreads), lds, stream, a);
+  hipLaunchKernelGGL(recurrence_combine_kernel, dim3(a.heads, num_entries, (a.N * a.P + 255) / 256),
+                     dim3(256), 0, stream, a);
+  hipLaunchKernelGGL((recurrence_kernel<NI, CPT, false, false, kRecOutput>), grid,
+                     dim3(kRecThreads), lds, stream, a);
 }
 
 template <int NI, int CPT>
@@ -264,13 +329,18 @@ static int launch_recurrence(const RecurrenceArgs& a, int num_entries, bool delt
 // `gates` [T, ldg] holds beta (heads; read by the delta rule only) and then the decays, one
 // per head or (`per_row`) one per head and row of S.  out [T, heads*P].  `max_q_len`: the
 // most tokens an entry brings (it chooses the launch's shape, never a result).
+// `num_chunks` 0: every entry is walked whole.  Else (without the delta rule) `chunks`
+// [num_chunks, 3] cuts every entry into runs of tokens (first, one past the last, entry), in
+// order, `entry_chunks` [B + 1] says which are whose, and chunk_state [num_chunks, heads, N,
+// P], chunk_decay [num_chunks, heads] are scratch.
 extern "C" int ts_linear_recurrence(const float* x, int ld, int q_col, int k_col, int v_col,
                                     const float* decay, const float* gates, int ldg, float* state,
                                     float* out, const int* positions, const int* entry_of_token,
                                     const int* q_start, const int* slot_ids, int num_tokens,
                                     int num_entries, int max_q_len, int heads, int kv_heads,
                                     int N, int P, int silu, int delta, int per_row,
-                                    hipStream_t stream) {
+                                    const int* chunks, const int* entry_chunks, int num_chunks,
+                                    float* chunk_state, float* chunk_decay, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || N <= 0 || P <= 0)
     TS_FAIL("linear_recurrence: bad sizes heads=%d kv_heads=%d dim=%d vdim=%d", heads, kv_heads, N, P);
@@ -287,8 +357,21 @@ extern "C" int ts_linear_recurrence(const float* x, int ld, int q_col, int k_col
     TS_FAIL("linear_recurrence: gates of %d columns are too few", ldg);
   RecurrenceArgs a{x, decay, gates, state, out,
                    BatchView{positions, entry_of_token, q_start, slot_ids},
-                   ld, q_col, k_col, v_col, ldg, heads, kv_heads, N, P, silu};
+                   ld, q_col, k_col, v_col, ldg, heads, kv_heads, N, P, silu,
+                   chunks, entry_chunks, chunk_state, chunk_decay};
   const int ni = (N + kRecSlices - 1) / kRecSlices;
+  if (num_chunks > 0) {
+    if (delta) TS_FAIL("linear_recurrence: the delta rule is not linear in S and runs whole");
+    if (!chunks || !entry_chunks || !chunk_state || !chunk_decay)
+      TS_FAIL("linear_recurrence: chunked without its lists and scratch");
+    if (ni > 16) TS_FAIL("linear_recurrence: chunks are built for up to 128 key channels");
+    if (ni <= 2) launch_recurrence_chunked<2, 4>(a, num_entries, num_chunks, stream);
+    else if (ni <= 4) launch_recurrence_chunked<4, 4>(a, num_entries, num_chunks, stream);
+    else if (ni <= 8) launch_recurrence_chunked<8, 4>(a, num_entries, num_chunks, stream);
+    else launch_recurrence_chunked<16, 4>(a, num_entries, num_chunks, stream);
+    TS_CHECK_LAUNCH("linear_recurrence (chunked)");
+    return 0;
+  }
   const int64_t wide_groups = (int64_t)heads * num_entries * ((P + 4 * kRecGroups - 1) / (4 * kRecGroups));
   const bool narrow = max_q_len >= 8 && wide_groups < 1024;
   int rc;

@@ -1061,18 +1061,9 @@ class HipOps:
         y = torch.empty(T, inner, dtype=torch.float32, device=self.device)
         # a step with a long portion runs its entries in chunks side by side (the lists are
         # the step's: every recurrent layer of the model uses the same)
-        chunks = entry_chunks = scratch = decays = None
-        num_chunks = 0
-        if batch.max_q_len > self.dispatch.scan_whole_tokens:
-            if "scan_chunks" not in batch.plans:
-                size, rows, firsts, t0 = self.lib.ts_ssm_scan_chunk(), [], [0], 0
-                for e, n in enumerate(batch.q_lens):
-                    rows += [(t0 + c, min(t0 + c + size, t0 + n), e) for c in range(0, n, size)]
-                    firsts.append(len(rows))
-                    t0 += n
-                batch.plans["scan_chunks"] = (self._upload_ints(rows), self._upload_ints(firsts),
-                                              len(rows))
-            chunks, entry_chunks, num_chunks = batch.plans["scan_chunks"]
+        chunks, entry_chunks, num_chunks = self._scan_chunks(batch)
+        scratch = decays = None
+        if num_chunks:
             scratch = torch.empty(num_chunks, heads, N, vdim, dtype=torch.float32,
                                   device=self.device)
             decays = torch.empty(num_chunks, heads, dtype=torch.float32, device=self.device)
@@ -1081,6 +1072,22 @@ class HipOps:
                    slots, T, batch.num_entries, heads, vdim, N, groups, _ptr(chunks),
                    _ptr(entry_chunks), num_chunks, _ptr(scratch), _ptr(decays), self._stream())
         return y
+
+    def _scan_chunks(self, batch):
+        """(chunk list, chunks of each entry, number of chunks) for a step with a portion long
+        enough to run in chunks side by side, else (None, None, 0).  The lists are the
+        step's: every recurrent layer of the model uses the same."""
+        if batch.max_q_len <= self.dispatch.scan_whole_tokens:
+            return None, None, 0
+        if "scan_chunks" not in batch.plans:
+            size, rows, firsts, t0 = self.lib.ts_ssm_scan_chunk(), [], [0], 0
+            for e, n in enumerate(batch.q_lens):
+                rows += [(t0 + c, min(t0 + c + size, t0 + n), e) for c in range(0, n, size)]
+                firsts.append(len(rows))
+                t0 += n
+            batch.plans["scan_chunks"] = (self._upload_ints(rows), self._upload_ints(firsts),
+                                          len(rows))
+        return batch.plans["scan_chunks"]
 
     def gated_group_norm(self, y, proj, norm_w, groups, eps, out_dtype):
         """(y * silu(z)) normalised in `groups` equal parts, times norm_w; z is the first
@@ -1142,11 +1149,21 @@ class HipOps:
             self._check("gates", gates, torch.float32, shape=(T, ldg))
         pos, eot, qs, slots = self._batch_ptrs(batch, T)
         out = torch.empty(T, heads * vdim, dtype=torch.float32, device=self.device)
+        # without the delta rule a long portion runs in chunks side by side
+        chunks = entry_chunks = scratch = decays = None
+        num_chunks = 0
+        if not delta and dim <= 128:
+            chunks, entry_chunks, num_chunks = self._scan_chunks(batch)
+        if num_chunks:
+            scratch = torch.empty(num_chunks, heads, dim, vdim, dtype=torch.float32,
+                                  device=self.device)
+            decays = torch.empty(num_chunks, heads, dtype=torch.float32, device=self.device)
         self._call(self.lib.ts_linear_recurrence, _ptr(x), ld, int(q_col), int(k_col), int(v_col),
                    _ptr(decay), _ptr(gates), ldg, _ptr(state), _ptr(out), pos, eot, qs, slots, T,
                    batch.num_entries, int(batch.max_q_len), heads, kv_heads, dim, vdim,
-                   int(bool(silu_inputs)),
-                   int(bool(delta)), int(bool(per_channel)), self._stream())
+                   int(bool(silu_inputs)), int(bool(delta)), int(bool(per_channel)),
+                   _ptr(chunks), _ptr(entry_chunks), num_chunks, _ptr(scratch), _ptr(decays),
+                   self._stream())
         return out
 
     def norm_gate(self, y, gate_rows, gate_col, norm_w, *, groups, gate, eps, out_dtype):

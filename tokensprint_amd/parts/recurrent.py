@@ -207,11 +207,23 @@ class SideBySide(Mixer):
     params: left, right (PartSpec of a mixer each), left_scale, right_scale."""
 
     def __init__(self, params, ctx):
+        self.left = self.right = None
         super().__init__(params, ctx)
         self.left = build_part(MIXERS, params["left"], ctx)
         self.right = build_part(MIXERS, params["right"], ctx)
         self.left_scale, self.right_scale = float(params["left_scale"]), float(params["right_scale"])
         self.capturable = self.left.capturable and self.right.capturable
+
+    @property
+    def ops(self):
+        return self._ops
+
+    @ops.setter
+    def ops(self, provider):          # whoever swaps the provider (a timer) swaps it for both
+        self._ops = provider
+        for side in (self.left, self.right):
+            if side is not None:
+                side.ops = provider
 
     def tensors(self):
         return {**self.left.tensors(), **self.right.tensors()}
