@@ -201,6 +201,10 @@ class TorchOps:
         if row is not None:
             resid.add_(row.float())
 
+    def stream_add_norm(self, resid, a, b, row, norm_w, eps, out_dtype):
+        self.stream_add(resid, a, b, row)
+        return self.rmsnorm(resid, norm_w, eps, out_dtype)
+
     def scaled_sum(self, a, scale_a, b, scale_b):
         return scale_a * a.float() + scale_b * b.float()
 

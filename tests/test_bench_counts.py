@@ -73,3 +73,22 @@ def test_compared_designs_are_of_equal_size():
         assert zono["width"] == qwen["hidden_size"] and zono["vocab"] == qwen["vocab_size"]
         assert len(zono["layers"]) == qwen["num_hidden_layers"]
         assert {e["type"] for e in zono["layers"]} == {"mamba2", "latent_attention"}
+
+
+def test_palelix_and_zonopel_are_compared_at_equal_size():
+    """`bench.py --compare-palelix` builds a Palelix and a Zonopel configuration per size with
+    the same width, depth, vocabulary and (within 2 %) number of parameters, every kind of
+    mixer and both kinds of feed-forward among the Palelix layers."""
+    import math
+
+    import bench
+    from tokensprint_amd.weights.random_init import declared_tensors
+    for name, size in bench.COMPARE_SIZES.items():
+        pale, zono = bench.palelix_configs(size)
+        count = [sum(math.prod(d.shape) for d in declared_tensors(raw).values())
+                 for raw in (pale, zono)]
+        assert abs(count[0] - count[1]) <= 0.02 * count[0], (name, count)
+        assert pale["width"] == zono["width"] and pale["vocab"] == zono["vocab"]
+        assert len(pale["layers"]) == len(zono["layers"])
+        assert {e["type"] for e in pale["layers"]} == {"delta", "lightning", "parallel"}
+        assert {e["mlp"]["kind"] for e in pale["layers"]} == {"dense", "moe"}

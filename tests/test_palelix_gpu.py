@@ -267,7 +267,7 @@ def test_expert_activation_and_stream_sums(gpu_device, dtype):
     got = ops.expert_activation(gate_up, weights, inner, 1.3, dtype)
     close(got, REF.expert_activation(gate_up, weights, inner, 1.3, dtype), **tol)
     assert (got.view(T, E, inner)[weights == 0] == 0).all()
-    for rows, width in ((1, 40), (9, 257)):
+    for rows, width in ((1, 40), (9, 257), (3, 2500)):
         resid = rnd((rows, width), 3).to(gpu_device)
         a, b = rnd((rows, width), 4).to(dtype).to(gpu_device), rnd((rows, width), 5).to(gpu_device)
         row = rnd((width,), 6).to(gpu_device)
@@ -276,6 +276,12 @@ def test_expert_activation_and_stream_sums(gpu_device, dtype):
             ops.stream_add(x, *args)
             REF.stream_add(y, *args)
             close(x, y)
+            w = (1 + 0.1 * rnd((width,), 7)).to(gpu_device)
+            if args[0] is not None:
+                x, y = resid.clone(), resid.clone()
+                close(ops.stream_add_norm(x, *args, w, 1e-5, dtype),
+                      REF.stream_add_norm(y, *args, w, 1e-5, dtype), **tol)
+                close(x, y)
         close(ops.scaled_sum(a, 0.7, b, -1.3), REF.scaled_sum(a, 0.7, b, -1.3))
         close(ops.take_columns(b, 3, width - 7, dtype), REF.take_columns(b, 3, width - 7, dtype), **tol)
 

@@ -30,6 +30,64 @@ extern "C" int ts_stream_add(float* resid, const void* a, int a_type, const void
   return 0;
 }
 
+// The same sum, and the RMS norm of the new stream: out = resid / sqrt(mean(resid^2) + eps) * w.
+// One workgroup a row; the row's values wait in registers between the two passes (up to
+// eight a thread), or are read back.
+template <typename TA, typename TB, typename TO>
+__global__ __launch_bounds__(256) void stream_add_norm_kernel(
+    float* __restrict__ resid, const TA* __restrict__ a, const TB* __restrict__ b,
+    const float* __restrict__ row, const float* __restrict__ w, TO* __restrict__ out, int width,
+    float eps) {
+  __shared__ float scratch[8];
+  constexpr int kKeep = 8;
+  const int64_t base = (int64_t)blockIdx.x * width;
+  float keep[kKeep], ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < kKeep; ++j) {
+    const int c = j * blockDim.x + threadIdx.x;
+    keep[j] = 0.f;
+    if (c < width) {
+      float v = resid[base + c];
+      v += b ? to_f32(a[base + c]) + to_f32(b[base + c]) : to_f32(a[base + c]);
+      if (row) v += row[c];
+      resid[base + c] = keep[j] = v;
+      ss = fmaf(v, v, ss);
+    }
+  }
+  for (int c = kKeep * blockDim.x + threadIdx.x; c < width; c += blockDim.x) {
+    float v = resid[base + c];
+    v += b ? to_f32(a[base + c]) + to_f32(b[base + c]) : to_f32(a[base + c]);
+    if (row) v += row[c];
+    resid[base + c] = v;
+    ss = fmaf(v, v, ss);
+  }
+  const float r = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+#pragma unroll
+  for (int j = 0; j < kKeep; ++j) {
+    const int c = j * blockDim.x + threadIdx.x;
+    if (c < width) out[base + c] = from_f32<TO>(keep[j] * r * w[c]);
+  }
+  for (int c = kKeep * blockDim.x + threadIdx.x; c < width; c += blockDim.x)
+    out[base + c] = from_f32<TO>(resid[base + c] * r * w[c]);
+}
+
+extern "C" int ts_stream_add_norm(float* resid, const void* a, int a_type, const void* b,
+                                  int b_type, const float* row, const float* w, void* out,
+                                  int out_type, int rows, int width, float eps,
+                                  hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (!a || !w || !out || width <= 0) TS_FAIL("stream_add_norm: a term, a weight and an output");
+  const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
+  TS_DISPATCH_TYPE(a_type, TA,
+    TS_DISPATCH_TYPE(b ? b_type : TS_F32, TB,
+      TS_DISPATCH_TYPE(out_type, TO,
+        hipLaunchKernelGGL((stream_add_norm_kernel<TA, TB, TO>), dim3(rows), dim3(threads), 0,
+                           stream, resid, (const TA*)a, (const TB*)b, row, w, (TO*)out, width,
+                           eps))));
+  TS_CHECK_LAUNCH("stream_add_norm");
+  return 0;
+}
+
 // out = sa * a + sb * b (float32 out).
 template <typename TA, typename TB>
 __global__ __launch_bounds__(256) void scaled_sum_kernel(

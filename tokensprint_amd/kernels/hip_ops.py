@@ -1235,6 +1235,25 @@ class HipOps:
                    _TYPE_CODE[b.dtype] if b is not None else 0, _ptr(row), resid.shape[0],
                    resid.shape[1], self._stream())
 
+    def stream_add_norm(self, resid, a, b, row, norm_w, eps, out_dtype):
+        """`stream_add(resid, a, b, row)` (b and row may be None), and the RMS norm (norm_w,
+        eps) of the new stream in `out_dtype`."""
+        self._check("resid", resid, torch.float32, ndim=2)
+        a = self._rows(a)
+        self._check("a", a, self._FLOATS, shape=resid.shape)
+        if b is not None:
+            b = self._rows(b)
+            self._check("b", b, self._FLOATS, shape=resid.shape)
+        if row is not None:
+            self._check("row", row, torch.float32, shape=(resid.shape[1],))
+        self._check("norm weight", norm_w, torch.float32, shape=(resid.shape[1],))
+        out = torch.empty(resid.shape, dtype=out_dtype, device=self.device)
+        self._call(self.lib.ts_stream_add_norm, _ptr(resid), _ptr(a), _TYPE_CODE[a.dtype], _ptr(b),
+                   _TYPE_CODE[b.dtype] if b is not None else 0, _ptr(row), _ptr(norm_w), _ptr(out),
+                   _TYPE_CODE[out_dtype], resid.shape[0], resid.shape[1], c_float(eps),
+                   self._stream())
+        return out
+
     def scaled_sum(self, a, scale_a, b, scale_b):
         """scale_a * a + scale_b * b -> float32."""
         a, b = self._rows(a), self._rows(b)

@@ -39,6 +39,31 @@ class PreparedRows:
     hint: NormHint
 
 
+@dataclass(frozen=True)
+class NormAhead:
+    """What a block whose sub-layers run side by side tells the block before it: the RMSNorm
+    (weight, eps) it opens with, and, where a row is to be added to the stream right in
+    front of it (`entering`), that row.  A block of the same kind in front may then add its
+    outputs (and the row) into the stream and take that norm in the same kernel."""
+
+    norm_weight: torch.Tensor
+    eps: float
+    row: torch.Tensor | None = None
+
+    def entering(self, row: torch.Tensor) -> "NormAhead":
+        return NormAhead(self.norm_weight, self.eps, row)
+
+
+@dataclass(frozen=True)
+class NormedRows:
+    """The stream summed up (nothing is left to add), with `rows`, its norm as the NormAhead
+    of the reader asked for it; `entered`: the reader's row is in the sum already.  Stands
+    where the stream's `delta` does, and only the block that gave the hint takes it."""
+
+    rows: torch.Tensor
+    entered: bool
+
+
 class UnmergedRows:
     """What `attend(defer_merge=True)` may return in place of a tensor: a decode step's
     attention output whose key splits have not been merged yet.  It is deliberately no

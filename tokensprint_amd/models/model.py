@@ -98,9 +98,14 @@ class Model:
             owner = r if run.cache_of is None else run.cache_of
             # what reads the stream after this run: the next run's block (the final norm
             # and the head take a plain delta)
-            next_hint = self.blocks[self.order[r + 1].layer].entry_hint() \
-                if r + 1 < len(self.order) and self.order[r + 1].enter is None else None
-            if run.enter is not None:
+            nxt = self.order[r + 1] if r + 1 < len(self.order) else None
+            next_hint = self.blocks[nxt.layer].entry_hint() if nxt is not None else None
+            if nxt is not None and nxt.enter is not None:
+                # a row enters in front of the next run: only a reader that can be told so
+                # may have its norm taken ahead
+                next_hint = next_hint.entering(self.enter_tables[nxt.enter[0]][nxt.enter[1]]) \
+                    if hasattr(next_hint, "entering") else None
+            if run.enter is not None and not getattr(delta, "entered", False):
                 # what is still to be added, then the row of this pass
                 ops.stream_add(resid, delta, None, self.enter_tables[run.enter[0]][run.enter[1]])
                 delta = None

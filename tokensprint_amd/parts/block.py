@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import torch
 
-from tokensprint_amd.kernels.stream import fused_rmsnorm_of
+from tokensprint_amd.kernels.stream import NormAhead, NormedRows, fused_rmsnorm_of
 from tokensprint_amd.parts.base import (BLOCKS, FEED_FORWARDS, FILTERS, MIXERS, NORMS, Block,
                                         StreamFilter, TensorDecl, SlotStateNeed, register)
 
@@ -106,16 +106,32 @@ class SandwichNormBlock(Block):
 class ParallelResidualBlock(Block):
     """One norm whose output both sub-layers read: with h = norm(x),
     x <- x + (mixer(h) + ffn(h)).  The feed-forward may be left out.  The stream leaves the
-    block summed up (no delta is handed on)."""
+    block summed up (no delta is handed on); where a block of this kind follows, the sum and
+    that block's norm (and a row that enters in front of it) are one kernel, and the normed
+    rows travel in delta's place."""
 
     ROLES = {"mixer_norm": (NORMS, True), "mixer": (MIXERS, True),
              "feed_forward": (FEED_FORWARDS, False)}
 
+    def entry_hint(self):
+        fused = fused_rmsnorm_of(self.mixer_norm)
+        if fused is None or not hasattr(self.ctx.ops, "stream_add_norm"):
+            return None
+        return NormAhead(fused[0], fused[1])
+
     def forward(self, resid, delta, batch, cache, write_cache, next_hint=None):
-        h = self.mixer_norm.forward(resid) if delta is None \
-            else self.mixer_norm.add_forward(resid, delta)
+        if isinstance(delta, NormedRows):
+            h = delta.rows
+        else:
+            h = self.mixer_norm.forward(resid) if delta is None \
+                else self.mixer_norm.add_forward(resid, delta)
         mixed = self.mixer.forward(h, batch, cache, write_cache)
         fed = self.feed_forward.forward(h, batch) if self.feed_forward is not None else None
+        if isinstance(next_hint, NormAhead):
+            rows = self.ctx.ops.stream_add_norm(resid, mixed, fed, next_hint.row,
+                                                next_hint.norm_weight, next_hint.eps,
+                                                self.ctx.dtype)
+            return resid, NormedRows(rows, next_hint.row is not None)
         self.ctx.ops.stream_add(resid, mixed, fed, None)
         return resid, None
 
