@@ -494,9 +494,11 @@ def test_float32_does_not_depend_on_the_cut(setup):
     a = drives.drive_whole(runner_for(model, page, 256 // page), requests)
     b = drives.drive_portions(runner_for(model, page, 256 // page), requests)
     c = drives.drive_mixed(runner_for(model, page, 480 // page), requests)
+    # (a long portion's recurrence adds a column's parts over sixteen lanes, a short one's over
+    # eight: the same sums in another order)
     for rid in requests:
-        torch.testing.assert_close(a.stacked(rid)[0], b.stacked(rid)[0], rtol=1e-4, atol=2e-5)
-        torch.testing.assert_close(a.stacked(rid)[0], c.stacked(rid)[0], rtol=1e-4, atol=2e-5)
+        torch.testing.assert_close(a.stacked(rid)[0], b.stacked(rid)[0], rtol=1e-4, atol=5e-5)
+        torch.testing.assert_close(a.stacked(rid)[0], c.stacked(rid)[0], rtol=1e-4, atol=5e-5)
 
 
 def plain_greedy(pcfg, w, prompt, n):

@@ -50,18 +50,21 @@ struct RecurrenceArgs {
 // (kRecOutput).  Twice the arithmetic, a sixty-fourth of the chain.
 constexpr int kRecWhole = 0, kRecLocal = 1, kRecOutput = 2;
 
-constexpr int kRecSlices = 8;              // lanes that share a column's dot products
 constexpr int kRecThreads = 128;
-constexpr int kRecGroups = kRecThreads / kRecSlices;   // 16 groups of columns a workgroup
 constexpr int kRecStage = 16;              // tokens staged in LDS at a time
 
-// Sum over the eight neighbouring lanes that share a column; every one of them gets it.  Two
-// exchanges inside a quad and one with the mirrored lane of the eight, all three in the
+// Sum over the eight or sixteen neighbouring lanes that share a column; every one of them
+// gets it.  Two exchanges inside a quad, one with the mirrored lane of the eight and one with
+// the lane eight further in the row of sixteen, all in the
 // vector pipeline (a shuffle through LDS costs a round trip each, on the recurrence's chain).
-__device__ __forceinline__ float sum8(float v) {
+template <int SL>
+__device__ __forceinline__ float sum_slices(float v) {
+  static_assert(SL == 8 || SL == 16, "eight or sixteen lanes share a column");
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true));
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true));
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true));
+  if (SL == 16)      // the other eight of a row of sixteen: rotated by eight
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, true));
   return v;
 }
 
@@ -79,23 +82,30 @@ __device__ __forceinline__ void read_rows(const float* p, float (&r)[NI]) {
   }
 }
 
-// A workgroup serves one (entry, head, 16 CPT columns of P) and walks the entry's tokens in
-// order.  Thread (cg, s) = (tid / 8, tid % 8) keeps rows [s NI, (s + 1) NI) of CPT columns in
-// registers; a column's dot products over the rows are added over the eight lanes that share
-// it, in one fixed order whatever CPT is, so the result does not depend on how a launch is
-// shaped.  Sixteen tokens' q, k, the workgroup's columns of v, and the gates are staged in
-// one of two LDS buffers (rows padded to 8 NI, so a thread's rows come in 16-byte reads)
-// while the sixteen before them are walked.
-template <int NI, int CPT, bool DELTA, bool PER_ROW, int MODE = kRecWhole>
+// A workgroup serves one (entry, head, 128 / SL x CPT columns of P) and walks the entry's
+// tokens in order.  Thread (cg, s) = (tid / SL, tid % SL) keeps rows [s NI, (s + 1) NI) of CPT
+// columns in registers; a column's dot products over the rows are added over the SL lanes
+// that share it.  Sixteen tokens' q, k, the workgroup's columns of v, and the gates are
+// staged in one of two LDS buffers (rows padded to SL NI, so a thread's rows come in 16-byte
+// reads) while the sixteen before them are walked.  A token's time is the chain of its
+// multiply-adds in one wavefront, so a long portion of few entries takes sixteen lanes a
+// column and one column a thread (half the rows a lane, twice the wavefronts), a step of
+// many entries eight lanes and four columns (its states stream in wider rows).
+template <int NI, int CPT, int SL, bool DELTA, bool PER_ROW, int MODE = kRecWhole>
 __global__ __launch_bounds__(kRecThreads) void recurrence_kernel(RecurrenceArgs a) {
+  constexpr int kRecSlices = SL, kRecGroups = kRecThreads / SL;
+  constexpr int EPT = kRecStage * SL * NI / kRecThreads;   // elements of q a thread stages
   extern __shared__ __align__(16) float lds[];
   constexpr int NP = kRecSlices * NI;                // padded rows
+  // a token's rows in LDS: the eight slices' runs of NI rows, 16 bytes between them, so that
+  // the eight 16-byte reads of an instruction fall into different banks
+  constexpr int SP = NI + 4, LP = kRecSlices * SP;
   constexpr int BC = kRecGroups * CPT;               // columns of the workgroup
-  constexpr int kQ = 0, kK = kRecStage * NP, kG = 2 * kRecStage * NP;
-  constexpr int kV = kG + kRecStage * (PER_ROW ? NP : 1);
+  constexpr int kQ = 0, kK = kRecStage * LP, kG = 2 * kRecStage * LP;
+  constexpr int kV = kG + kRecStage * (PER_ROW ? LP : 1);
   constexpr int kB = kV + kRecStage * BC;
   constexpr int kBuf = (kB + kRecStage + 3) / 4 * 4;
-  constexpr int VPT = kRecStage * BC / kRecThreads;  // values of v a thread stages: 2 CPT
+  constexpr int VPT = kRecStage * BC / kRecThreads;  // values of v a thread stages
   const int N = a.N;
   const int h = blockIdx.x;
   const int s = threadIdx.x % kRecSlices, cg = threadIdx.x / kRecSlices;
@@ -131,16 +141,18 @@ __global__ __launch_bounds__(kRecThreads) void recurrence_kernel(RecurrenceArgs 
   __syncthreads();
 
   // a stage's operands: from memory into registers (fetch), from there into a buffer (commit)
-  float pq[NI], pk[NI], pg[PER_ROW ? NI : 1], pv[VPT], pbeta = 0.f, pgate = 1.f;
+  float pq[EPT], pk[EPT], pg[PER_ROW ? EPT : 1], pv[VPT], pbeta = 0.f, pgate = 1.f;
   auto fetch = [&](int t0) {
     const int nt = min(kRecStage, end - t0);
+    // (element j of a thread is row i % NP of token i / NP in the padded layout: NP is a
+    // power of two, so no division by a size only known at run time)
 #pragma unroll
-    for (int j = 0; j < NI; ++j) {
+    for (int j = 0; j < EPT; ++j) {
       const int i = j * kRecThreads + threadIdx.x;
-      const int tt = i / N, n = i - tt * N;
+      const int tt = i / NP, n = i % NP;
       pq[j] = pk[j] = 0.f;
       if (PER_ROW) pg[j] = 0.f;
-      if (tt < nt) {
+      if (tt < nt && n < N) {
         const float* row = a.x + (int64_t)(t0 + tt) * a.ld;
         pq[j] = row[a.q_col + hk * N + n];
         pk[j] = row[a.k_col + hk * N + n];
@@ -162,14 +174,12 @@ __global__ __launch_bounds__(kRecThreads) void recurrence_kernel(RecurrenceArgs 
   };
   auto commit = [&](float* buf) {
 #pragma unroll
-    for (int j = 0; j < NI; ++j) {
-      const int i = j * kRecThreads + threadIdx.x;
-      const int tt = i / N, n = i - tt * N;
-      if (tt < kRecStage) {
-        buf[kQ + tt * NP + n] = a.silu ? silu_f(pq[j]) : pq[j];
-        buf[kK + tt * NP + n] = a.silu ? silu_f(pk[j]) : pk[j];
-        if (PER_ROW) buf[kG + tt * NP + n] = pg[j];
-      }
+    for (int j = 0; j < EPT; ++j) {
+      const int i = j * kRecThreads + threadIdx.x;       // = token * NP + row, padding included
+      const int at = (i / NP) * LP + (i % NP) / NI * SP + i % NI;
+      buf[kQ + at] = a.silu ? silu_f(pq[j]) : pq[j];
+      buf[kK + at] = a.silu ? silu_f(pk[j]) : pk[j];
+      if (PER_ROW) buf[kG + at] = pg[j];
     }
 #pragma unroll
     for (int j = 0; j < VPT; ++j)
@@ -190,14 +200,15 @@ __global__ __launch_bounds__(kRecThreads) void recurrence_kernel(RecurrenceArgs 
     if (more) fetch(t0 + kRecStage);
     const float* buf = lds + which * kBuf;
     for (int tt = 0; tt < nt; ++tt) {
-      float kr[NI], u[CPT], acc[CPT];
-      read_rows<NI>(buf + kK + tt * NP + s * NI, kr);
+      float kr[NI], qr[NI], u[CPT], acc[CPT];
+      read_rows<NI>(buf + kK + tt * LP + s * SP, kr);
+      if (MODE != kRecLocal) read_rows<NI>(buf + kQ + tt * LP + s * SP, qr);   // one trip to LDS a token
 #pragma unroll
       for (int c = 0; c < CPT; ++c) u[c] = buf[kV + tt * BC + cg * CPT + c];
       const float g_all = PER_ROW ? 1.f : buf[kG + tt];
       if (DELTA) {
         float gr[NI];
-        if constexpr (PER_ROW) read_rows<NI>(buf + kG + tt * NP + s * NI, gr);
+        if constexpr (PER_ROW) read_rows<NI>(buf + kG + tt * LP + s * SP, gr);
         float pred[CPT][2];
 #pragma unroll
         for (int c = 0; c < CPT; ++c) pred[c][0] = pred[c][1] = 0.f;
@@ -212,7 +223,7 @@ __global__ __launch_bounds__(kRecThreads) void recurrence_kernel(RecurrenceArgs 
         }
         const float beta = buf[kB + tt];
 #pragma unroll
-        for (int c = 0; c < CPT; ++c) u[c] = beta * (u[c] - sum8(pred[c][0] + pred[c][1]));
+        for (int c = 0; c < CPT; ++c) u[c] = beta * (u[c] - sum_slices<SL>(pred[c][0] + pred[c][1]));
 #pragma unroll
         for (int i = 0; i < NI; ++i)
 #pragma unroll
@@ -227,8 +238,6 @@ __global__ __launch_bounds__(kRecThreads) void recurrence_kernel(RecurrenceArgs 
         total_decay *= g_all;
         continue;
       }
-      float qr[NI];
-      read_rows<NI>(buf + kQ + tt * NP + s * NI, qr);
 #pragma unroll
       for (int c = 0; c < CPT; ++c) {
         float a0 = 0.f, a1 = 0.f;
@@ -237,7 +246,7 @@ __global__ __launch_bounds__(kRecThreads) void recurrence_kernel(RecurrenceArgs 
           a0 = fmaf(S[i][c], qr[i], a0);
           a1 = fmaf(S[i + 1][c], qr[i + 1], a1);
         }
-        acc[c] = sum8(a0 + a1);
+        acc[c] = sum_slices<SL>(a0 + a1);
         if (s == 0 && p0 + c < a.P) a.out[(int64_t)(t0 + tt) * inner + h * a.P + p0 + c] = acc[c];
       }
     }
@@ -278,50 +287,55 @@ __global__ __launch_bounds__(256) void recurrence_combine_kernel(RecurrenceArgs 
 template <int NI, int CPT>
 static void launch_recurrence_chunked(const RecurrenceArgs& a, int num_entries, int num_chunks,
                                       hipStream_t stream) {
-  constexpr int NP = kRecSlices * NI, BC = kRecGroups * CPT;
+  constexpr int SL = 8, LP = SL * (NI + 4), BC = kRecThreads / SL * CPT;
   const dim3 grid(a.heads, num_chunks, (a.P + BC - 1) / BC);
-  const int buf = (kRecStage * (2 * NP + 1 + BC + 1) + 3) / 4 * 4;
+  const int buf = (kRecStage * (2 * LP + 1 + BC + 1) + 3) / 4 * 4;
   const size_t lds = (size_t)2 * buf * sizeof(float);
-  hipLaunchKernelGGL((recurrence_kernel<NI, CPT, false, false, kRecLocal>), grid,
+  hipLaunchKernelGGL((recurrence_kernel<NI, CPT, 8, false, false, kRecLocal>), grid,
                      dim3(kRecThreads), lds, stream, a);
   hipLaunchKernelGGL(recurrence_combine_kernel, dim3(a.heads, num_entries, (a.N * a.P + 255) / 256),
                      dim3(256), 0, stream, a);
-  hipLaunchKernelGGL((recurrence_kernel<NI, CPT, false, false, kRecOutput>), grid,
+  hipLaunchKernelGGL((recurrence_kernel<NI, CPT, 8, false, false, kRecOutput>), grid,
                      dim3(kRecThreads), lds, stream, a);
 }
 
-template <int NI, int CPT>
+template <int NI, int CPT, int SL>
 static int launch_recurrence_cols(const RecurrenceArgs& a, int num_entries, bool delta, bool per_row,
                                   hipStream_t stream) {
-  constexpr int NP = kRecSlices * NI, BC = kRecGroups * CPT;
+  constexpr int LP = SL * (NI + 4), BC = kRecThreads / SL * CPT;
   const dim3 grid(a.heads, num_entries, (a.P + BC - 1) / BC);
   const dim3 block(kRecThreads);
-  const int buf = (kRecStage * (2 * NP + (per_row ? NP : 1) + BC + 1) + 3) / 4 * 4;
+  const int buf = (kRecStage * (2 * LP + (per_row ? LP : 1) + BC + 1) + 3) / 4 * 4;
   const size_t lds = (size_t)2 * buf * sizeof(float);
-  const void* fn = delta && per_row ? (const void*)recurrence_kernel<NI, CPT, true, true>
-                   : delta          ? (const void*)recurrence_kernel<NI, CPT, true, false>
-                                    : (const void*)recurrence_kernel<NI, CPT, false, false>;
+  const void* fn = delta && per_row ? (const void*)recurrence_kernel<NI, CPT, SL, true, true>
+                   : delta          ? (const void*)recurrence_kernel<NI, CPT, SL, true, false>
+                                    : (const void*)recurrence_kernel<NI, CPT, SL, false, false>;
   if (lds > 64 * 1024 &&
       hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
     return -1;
   if (delta && per_row)
-    hipLaunchKernelGGL((recurrence_kernel<NI, CPT, true, true>), grid, block, lds, stream, a);
+    hipLaunchKernelGGL((recurrence_kernel<NI, CPT, SL, true, true>), grid, block, lds, stream, a);
   else if (delta)
-    hipLaunchKernelGGL((recurrence_kernel<NI, CPT, true, false>), grid, block, lds, stream, a);
+    hipLaunchKernelGGL((recurrence_kernel<NI, CPT, SL, true, false>), grid, block, lds, stream, a);
   else
-    hipLaunchKernelGGL((recurrence_kernel<NI, CPT, false, false>), grid, block, lds, stream, a);
+    hipLaunchKernelGGL((recurrence_kernel<NI, CPT, SL, false, false>), grid, block, lds, stream, a);
   return 0;
 }
 
-// Four columns a thread where the launch has workgroups enough without (a step of many
-// entries streams its states in wider rows); one column a thread where a few entries' long
-// portions are walked, which is then sixteen times the workgroups and a quarter of the
-// chain a token.
-template <int NI>
+// `ni8`: rows a lane keeps when eight lanes share a column (a power of two from 2 to 32).
+// Eight lanes and four columns a thread where the launch has workgroups enough (a step of many
+// entries streams its states in wider rows); sixteen lanes and one column a thread where a few
+// entries' long portions are walked.
+template <int NI8>
 static int launch_recurrence(const RecurrenceArgs& a, int num_entries, bool delta, bool per_row,
                              bool narrow, hipStream_t stream) {
-  return narrow ? launch_recurrence_cols<NI, 1>(a, num_entries, delta, per_row, stream)
-                : launch_recurrence_cols<NI, 4>(a, num_entries, delta, per_row, stream);
+  if (narrow)
+    return launch_recurrence_cols<(NI8 >= 4 ? NI8 / 2 : 2), 1, 16>(a, num_entries, delta, per_row,
+                                                                  stream);
+  if constexpr (NI8 <= 16)
+    return launch_recurrence_cols<NI8, 4, 8>(a, num_entries, delta, per_row, stream);
+  else        // (four columns of 32 rows a thread do not fit the registers)
+    return launch_recurrence_cols<NI8, 1, 8>(a, num_entries, delta, per_row, stream);
 }
 
 // x [T, ld] float32 holds q, k (kv_heads x N each) and v (heads x P) at the given columns
@@ -344,8 +358,7 @@ extern "C" int ts_linear_recurrence(const float* x, int ld, int q_col, int k_col
   if (num_tokens <= 0) return 0;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || N <= 0 || P <= 0)
     TS_FAIL("linear_recurrence: bad sizes heads=%d kv_heads=%d dim=%d vdim=%d", heads, kv_heads, N, P);
-  if (N > kRecSlices * 32)
-    TS_FAIL("linear_recurrence: %d key channels, at most %d are built", N, kRecSlices * 32);
+  if (N > 256) TS_FAIL("linear_recurrence: %d key channels, at most 256 are built", N);
   if (q_col < 0 || k_col < 0 || v_col < 0 || q_col + kv_heads * N > ld || k_col + kv_heads * N > ld ||
       v_col + heads * P > ld)
     TS_FAIL("linear_recurrence: columns outside the rows (ld=%d)", ld);
@@ -359,7 +372,7 @@ extern "C" int ts_linear_recurrence(const float* x, int ld, int q_col, int k_col
                    BatchView{positions, entry_of_token, q_start, slot_ids},
                    ld, q_col, k_col, v_col, ldg, heads, kv_heads, N, P, silu,
                    chunks, entry_chunks, chunk_state, chunk_decay};
-  const int ni = (N + kRecSlices - 1) / kRecSlices;
+  const int ni = (N + 7) / 8;
   if (num_chunks > 0) {
     if (delta) TS_FAIL("linear_recurrence: the delta rule is not linear in S and runs whole");
     if (!chunks || !entry_chunks || !chunk_state || !chunk_decay)
@@ -372,14 +385,14 @@ extern "C" int ts_linear_recurrence(const float* x, int ld, int q_col, int k_col
     TS_CHECK_LAUNCH("linear_recurrence (chunked)");
     return 0;
   }
-  const int64_t wide_groups = (int64_t)heads * num_entries * ((P + 4 * kRecGroups - 1) / (4 * kRecGroups));
+  const int64_t wide_groups = (int64_t)heads * num_entries * ((P + 63) / 64);
   const bool narrow = max_q_len >= 8 && wide_groups < 1024;
   int rc;
   if (ni <= 2) rc = launch_recurrence<2>(a, num_entries, delta, per_row, narrow, stream);
   else if (ni <= 4) rc = launch_recurrence<4>(a, num_entries, delta, per_row, narrow, stream);
   else if (ni <= 8) rc = launch_recurrence<8>(a, num_entries, delta, per_row, narrow, stream);
   else if (ni <= 16) rc = launch_recurrence<16>(a, num_entries, delta, per_row, narrow, stream);
-  else rc = launch_recurrence<32>(a, num_entries, delta, per_row, true, stream);   // (registers)
+  else rc = launch_recurrence<32>(a, num_entries, delta, per_row, narrow, stream);
   if (rc != 0) TS_FAIL("linear_recurrence: %d key channels need more LDS than the device gives", N);
   TS_CHECK_LAUNCH("linear_recurrence");
   return 0;
