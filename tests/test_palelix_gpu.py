@@ -423,15 +423,21 @@ def compare(col, ref, rtol, atol):
     that is lost puts every later row outside."""
     if rtol < 1e-2:
         return drives.compare(col, ref, rtol, atol)
-    rows = bad = 0
+    errors = []
     for rid, want in ref.items():
         got, positions = col.stacked(rid)
         assert positions == list(range(want.shape[0]))
         assert torch.isfinite(got).all()
-        wrong = ~((got - want).abs() <= drives.row_tolerance(want, rtol, atol))
-        rows += want.shape[0]
-        bad += int(wrong.any(dim=1).sum())
-    assert bad <= 0.04 * rows, f"{bad} of {rows} rows outside the tolerance"
+        # a row's error as the replayed traces are judged: the root mean square of the
+        # difference over the vocabulary, its mean taken off, in units of the logits' own
+        diff = got - want
+        diff = diff - diff.mean(dim=1, keepdim=True)
+        errors.append(diff.pow(2).mean(dim=1).sqrt() / want.std())
+    errors = torch.cat(errors)
+    bad = int((errors > atol).sum())
+    assert bad <= 0.04 * errors.numel() and float(errors.median()) < atol / 3, \
+        (f"{bad} of {errors.numel()} rows outside the tolerance; median error "
+         f"{float(errors.median()):.4f}, largest {float(errors.max()):.4f}")
 
 
 @pytest.fixture(scope="module", params=[(n, d) for n in sorted(PALE)
@@ -499,6 +505,37 @@ def test_float32_does_not_depend_on_the_cut(setup):
     for rid in requests:
         torch.testing.assert_close(a.stacked(rid)[0], b.stacked(rid)[0], rtol=1e-4, atol=5e-5)
         torch.testing.assert_close(a.stacked(rid)[0], c.stacked(rid)[0], rtol=1e-4, atol=5e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
+def test_layer_shapes_of_a_real_model(gpu_device, tmp_path, dtype):
+    """Heads of 128 x 128, a width of 512, experts of 256: the instantiations and products
+    that the tiny configurations do not reach (sixteen rows a lane, the vendor library's
+    products, attention heads of 128), whole, in portions and decoded."""
+    from helpers import (palelix_config, palelix_delta, palelix_delta_sizes, palelix_dense,
+                         palelix_lightning, palelix_moe, palelix_parallel)
+    # (bfloat16: every expert is used, so that no choice between nearly equal scores is
+    # decided by rounding and the comparison shows the kernels' precision alone)
+    moe = palelix_moe(ff=256, limit=7.0, experts=8, top=2, count=4, keep=2) \
+        if dtype == torch.float32 else \
+        palelix_moe(ff=256, limit=7.0, experts=8, top=8, count=1, keep=1)
+    cfg = palelix_config(width=512, vocab=1000, eps=1e-6, loop=(1, 3, 2), layers=[
+        palelix_delta(heads=4, kv_heads=2, dim=128, vdim=128, conv=4, mlp=palelix_dense(1024)),
+        palelix_lightning(heads=4, dim=128, vdim=128, decay=(0.75, 0.9, 0.99, 0.999), mlp=moe),
+        palelix_parallel(heads=4, kv_heads=2, dim=128, vdim=128, rot_dims=64, base=1e6,
+                         scale=128 ** -0.5, left_scale=1.0, right_scale=1.0,
+                         right=palelix_delta_sizes(heads=2, kv_heads=2, dim=64, vdim=128, conv=4,
+                                                   ranks=(64, 64)), mlp=moe)])
+    d = write_palelix_model(tmp_path, cfg, 5, dtype, std=0.04, sharpen=1.0)
+    pcfg, w = plain.read_model_dir(d)
+    _, model = load_model(d, dtype, gpu_device)
+    requests = {"a": random_prompt(150, 1000, 1), "b": random_prompt(37, 1000, 2)}
+    ref = {rid: plain.forward(pcfg, w, t).float() for rid, t in requests.items()}
+    rtol, atol = TOL[dtype]
+    compare(drives.drive_whole(runner_for(model, 16, 24), requests), ref, rtol, atol)
+    compare(drives.drive_prefill_then_decode(runner_for(model, 16, 24), requests, tail=20),
+            ref, rtol, atol)
+    compare(drives.drive_portions(runner_for(model, 16, 24), requests), ref, rtol, atol)
 
 
 def plain_greedy(pcfg, w, prompt, n):
